@@ -1,0 +1,156 @@
+/* C ABI of the MI355X (gfx950) transducer-loss kernels.
+ *
+ * The reference exposes this path as a pybind11 function that takes torch
+ * tensors (optimized_transducer/python/csrc/optimized_transducer.cc:12-19) and
+ * keeps its CUDA launchers private to one translation unit
+ * (optimized_transducer/csrc/cuda.cu).  This header is the same set of steps
+ * with plain pointers and sizes, so that any host language can bind it; the
+ * torch extension `_optimized_transducer` of this repository is one such
+ * binding and adds nothing but argument checks and allocation.
+ *
+ * Conventions
+ *   - every pointer is DEVICE memory on the current HIP device unless stated;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     work is enqueued, nothing here synchronises;
+ *   - packed layout (reference README.md:133-136): utterance b owns rows
+ *     [row_splits[b], row_splits[b+1]) of every per-row array; inside it cell
+ *     (t, u), 0 <= t < T_b, 0 <= u <= U_b, is row row_splits[b] + t*(U_b+1) + u;
+ *   - return value: 0 on success, a positive hipError_t from the launch, or a
+ *     negative OT_E_* code for arguments the kernels cannot run with.
+ */
+#ifndef OT_TRANSDUCER_H_
+#define OT_TRANSDUCER_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OT_E_BAD_ARG (-1)       /* null pointer / non-positive size            */
+#define OT_E_TOO_LONG (-2)      /* max(U)+1 exceeds OT_MAX_U1                  */
+#define OT_E_MISALIGNED (-3)    /* logits / grad not 4-byte aligned            */
+
+/* Largest U+1 the lattice kernels handle (one thread per u, one workgroup per
+ * utterance and direction).  The reference's CUDA path has the same bound
+ * (cuda.cu:10, cuda.cu:202). */
+#define OT_MAX_U1 1024
+
+/* Batch facts gathered on the device by ot_row_splits; the host-side argument
+ * checks of the reference (transducer-loss.cc:49-66) need exactly these and
+ * obtain them with three blocking .item() calls.  32 bytes. */
+typedef struct ot_batch_status {
+  int64_t sum_tu;          /* sum_b T_b * (U_b + 1), exact in 64 bits          */
+  int32_t targets_max;     /* max over the whole (N, targets_cols) array       */
+  int32_t targets_min;     /* min over the same array                          */
+  int32_t target_len_max;  /* max_b U_b                                        */
+  int32_t target_len_min;  /* min_b U_b                                        */
+  int32_t logit_len_max;   /* max_b T_b                                        */
+  int32_t logit_len_min;   /* min_b T_b                                        */
+} ot_batch_status;
+
+/* Row offsets + batch facts in one launch.
+ * Replaces the ATen sequence sizes = T*(U+1); cumsum(int32); cat(zero) at
+ * cuda.cu:411-414 and the reductions at transducer-loss.cc:49,53,62.
+ * row_splits: (N+1,) int32, row_splits[0] = 0, int32 wrap-around like the
+ * reference; status: one ot_batch_status.  targets may be NULL when
+ * targets_cols == 0. */
+int ot_row_splits(const int32_t *logit_lengths, const int32_t *target_lengths,
+                  const int32_t *targets, int32_t N, int32_t targets_cols,
+                  int32_t *row_splits, ot_batch_status *status, void *stream);
+
+/* Row -> utterance map, (rows,) int32.  Replaces RowSplitsToRowIds /
+ * mgpu::load_balance_search (cuda.cu:40-59).  The kernels below do not need
+ * it (they decode rows from row_splits); it exists for callers and tests. */
+int ot_row_ids(const int32_t *row_splits, int32_t N, int64_t rows,
+               int32_t *row_ids, void *stream);
+
+/* Per-row denominators and blank/symbol log-probabilities.
+ * from_log_softmax == 0: den[r] = logsumexp(logits[r, :]) (the ATen call at
+ *   cuda.cu:427), lp[r] = {logits[r,blank]-den[r], logits[r,target_u]-den[r]}
+ *   (ComputeLogProbs, cuda.cu:71-97 / kernels.cu:30-60); one fused kernel that
+ *   reads each row once.
+ * from_log_softmax != 0: den is not touched (may be NULL) and lp holds the two
+ *   gathered values as they are (ComputeLogProbsForLogSoftmax, cuda.cu:111-133).
+ * lp is (rows, 2) float; lp[r][1] at u == U_b, which the reference leaves
+ * uninitialised, is written as -inf.  Rows beyond row_splits[N] (only possible
+ * when the caller's sizes are inconsistent) get den only. */
+int ot_log_probs(const float *logits, const int32_t *targets,
+                 const int32_t *target_lengths, const int32_t *row_splits,
+                 int32_t N, int32_t targets_cols, int64_t rows, int32_t V,
+                 int32_t blank, int32_t from_log_softmax, float *den, float *lp,
+                 void *stream);
+
+/* Forward and backward lattice variables, both directions in one launch.
+ * Replaces ComputeAlpha / ComputeBeta and their one-symbol-per-frame twins
+ * (cuda.cu:162-306, kernels.cu:200-313, kernels.cu:415-519).
+ * alpha, beta: (rows,) float.  scores_alpha[b] = alpha(T-1,U)+lp(T-1,U).blank,
+ * scores_beta[b] = beta(0,0); both are log-likelihoods.  Cells outside the
+ * band of the one-symbol-per-frame lattice (uninitialised in the reference)
+ * are -inf.  max_u1 = max_b(U_b)+1 sizes the workgroup; must be <= OT_MAX_U1. */
+int ot_alpha_beta(const float *lp, const int32_t *logit_lengths,
+                  const int32_t *target_lengths, const int32_t *row_splits,
+                  int32_t N, int32_t max_u1, int32_t one_sym_per_frame,
+                  float *alpha, float *beta, float *scores_alpha,
+                  float *scores_beta, void *stream);
+
+/* Gradient of the negative log-likelihood w.r.t. the rows of `logits`, times
+ * grad_scale.
+ * from_log_softmax == 0: ComputeGradient / ComputeGradientOneSymPerFrame
+ *   (cuda.cu:308-346, kernels.cu:522-651); `grad` may be the same pointer as
+ *   `logits` (the reference's in-place mode, cuda.cu:449) - each row is read
+ *   completely before it is written.  lp is not used (may be NULL).
+ * from_log_softmax != 0: ComputeGradientForLogSoftmax(+OneSymPerFrame)
+ *   (cuda.cu:364-400, kernels.cu:653-779); `grad` must not alias `logits`;
+ *   only lp is read, logits and den may be NULL.
+ * An utterance whose beta(0,0) is not finite gets an all-zero gradient
+ * (kernels.cu:558-563).  grad_scale = 1 reproduces the reference; 1/N folds
+ * the `grad /= N` of reduction="mean" (transducer_loss.py:150). */
+int ot_gradient(const float *logits, const float *lp, const float *den,
+                const float *alpha, const float *beta, const int32_t *targets,
+                const int32_t *logit_lengths, const int32_t *target_lengths,
+                const int32_t *row_splits, int32_t N, int32_t targets_cols,
+                int64_t rows, int32_t V, int32_t blank,
+                int32_t from_log_softmax, int32_t one_sym_per_frame,
+                float grad_scale, float *grad, void *stream);
+
+/* In-place x *= *factor for n floats, skipped entirely on the device when
+ * *factor == 1.  Replaces ctx.grad.mul_(loss_grad) in backward
+ * (transducer_loss.py:162) without a host read of loss_grad. */
+int ot_scale_by_device_scalar(float *x, int64_t n, const float *factor,
+                              void *stream);
+
+/* Bytes of device scratch ot_transducer_loss needs for N utterances and
+ * `rows` packed rows. */
+size_t ot_workspace_bytes(int32_t N, int64_t rows);
+
+/* The whole path on one stream, no host synchronisation:
+ * row_splits -> log_probs -> alpha_beta -> gradient (ComputeTransducerLossCuda,
+ * cuda.cu:402-457).  scores: (N,) log-likelihoods from alpha.  grad may be
+ * NULL (forward only), equal to logits (in place, logits input only) or a
+ * separate (rows, V) buffer.  `status` receives the batch facts; the caller
+ * is responsible for checking them (sum_tu == rows, targets_max < V, ...)
+ * BEFORE calling when the inputs are untrusted, e.g. with ot_row_splits.
+ * max_u1 must equal max_b(U_b)+1. */
+int ot_transducer_loss(const float *logits, const int32_t *targets,
+                       const int32_t *logit_lengths,
+                       const int32_t *target_lengths, int32_t N,
+                       int32_t targets_cols, int64_t rows, int32_t V,
+                       int32_t blank, int32_t from_log_softmax,
+                       int32_t one_sym_per_frame, int32_t max_u1,
+                       float grad_scale, void *workspace,
+                       size_t workspace_bytes, float *scores, float *grad,
+                       ot_batch_status *status, void *stream);
+
+/* Plain device-to-device copy kernel of n floats; used to calibrate profiler
+ * byte counters against a transfer of known size. */
+int ot_copy_floats(const float *src, float *dst, int64_t n, void *stream);
+
+/* Text for a return value of the functions above. */
+const char *ot_error_string(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OT_TRANSDUCER_H_ */

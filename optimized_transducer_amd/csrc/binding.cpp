@@ -1,0 +1,297 @@
+// Torch extension `_optimized_transducer`: the drop-in for the reference's
+// pybind11 module (optimized_transducer/python/csrc/optimized_transducer.cc:12-19)
+// and its argument checks / dispatch (optimized_transducer/csrc/transducer-loss.cc:21-96).
+//
+// This file only checks arguments, allocates through torch's caching allocator
+// and enqueues the C-ABI kernels of include/ot_transducer.h on torch's current
+// HIP stream.  There is no CPU implementation behind it: CPU tensors are
+// checked like the reference checks them and then rejected.
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+#include <torch/extension.h>
+
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "ot_transducer.h"
+
+namespace {
+
+void check_hip(hipError_t e, const char *file, int line) {
+  if (e != hipSuccess) {
+    std::ostringstream os;
+    os << file << ":" << line << ": " << hipGetErrorString(e) << "\n";
+    throw std::runtime_error(os.str());
+  }
+}
+void check_ot(int rc, const char *file, int line) {
+  if (rc != 0) {
+    std::ostringstream os;
+    os << file << ":" << line << ": " << ot_error_string(rc) << "\n";
+    throw std::runtime_error(os.str());
+  }
+}
+#define OT_CHECK_HIP(x) check_hip((x), __FILE__, __LINE__)
+#define OT_CHECK(x) check_ot((x), __FILE__, __LINE__)
+
+// ---- optional per-kernel timing (hipEvents on the launch stream) ------------
+struct Timed {
+  std::string name;
+  hipEvent_t start, stop;
+};
+std::mutex g_prof_mutex;
+bool g_profiling = false;
+std::vector<Timed> g_timed;
+
+struct ScopedTimer {
+  hipStream_t stream;
+  Timed t;
+  bool on;
+  ScopedTimer(const char *name, hipStream_t s) : stream(s), on(g_profiling) {
+    if (!on) return;
+    t.name = name;
+    OT_CHECK_HIP(hipEventCreate(&t.start));
+    OT_CHECK_HIP(hipEventCreate(&t.stop));
+    OT_CHECK_HIP(hipEventRecord(t.start, stream));
+  }
+  ~ScopedTimer() {
+    if (!on) return;
+    (void)hipEventRecord(t.stop, stream);
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    g_timed.push_back(t);
+  }
+};
+
+void set_profiling(bool on) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  g_profiling = on;
+}
+
+// Returns [(kernel name, milliseconds)] recorded since the last call; blocks
+// until the recorded events have completed.
+std::vector<std::pair<std::string, double>> take_profile() {
+  std::vector<Timed> timed;
+  {
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    timed.swap(g_timed);
+  }
+  std::vector<std::pair<std::string, double>> out;
+  for (auto &t : timed) {
+    float ms = 0.f;
+    OT_CHECK_HIP(hipEventSynchronize(t.stop));
+    OT_CHECK_HIP(hipEventElapsedTime(&ms, t.start, t.stop));
+    out.emplace_back(t.name, (double)ms);
+    (void)hipEventDestroy(t.start);
+    (void)hipEventDestroy(t.stop);
+  }
+  return out;
+}
+
+// ---- the value checks of transducer-loss.cc:49-66, given the batch facts ----
+void check_batch_values(const torch::Tensor &logits, const torch::Tensor &targets,
+                        int64_t sum_all_TU, int64_t targets_max, int64_t target_len_max,
+                        int32_t blank) {
+  torch::CheckedFrom checked_from = "ComputeTransducerLoss";
+  torch::checkSize(checked_from, torch::TensorArg(logits, "logits", 0), 0, sum_all_TU);
+  TORCH_CHECK(targets_max < logits.size(1), "targets.max() vs logits.size(1) is ", targets_max,
+              " vs ", logits.size(1), ". Expect targets.max() < logits.size(1)");
+  TORCH_CHECK((0 <= blank && blank < logits.size(1)), "blank vs logits.size(1) is ", blank,
+              " vs ", logits.size(1), ". Expect 0 <= blank < logits.size(1)");
+  TORCH_CHECK((targets.size(1) == target_len_max),
+              "targets.size(1) should be equal to target_lengths.max().",
+              "But targets.size(1) is ", targets.size(1), ", and target_lengths.max() is ",
+              target_len_max);
+}
+
+inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
+    torch::Tensor &logits, const torch::Tensor &targets, const torch::Tensor &logit_lengths,
+    const torch::Tensor &target_lengths, int32_t blank, bool from_log_softmax,
+    bool one_sym_per_frame, double grad_scale) {
+  auto logits_arg = torch::TensorArg(logits, "logits", 0);
+  auto targets_arg = torch::TensorArg(targets, "targets", 1);
+  auto logit_lengths_arg = torch::TensorArg(logit_lengths, "logit_lengths", 2);
+  auto target_lengths_arg = torch::TensorArg(target_lengths, "target_lengths", 3);
+  torch::CheckedFrom checked_from = "ComputeTransducerLoss";
+
+  // transducer-loss.cc:33-46, same order
+  torch::checkScalarType(checked_from, logits_arg, torch::kFloat);
+  torch::checkScalarType(checked_from, targets_arg, torch::kInt32);
+  torch::checkScalarType(checked_from, logit_lengths_arg, torch::kInt32);
+  torch::checkScalarType(checked_from, target_lengths_arg, torch::kInt32);
+  torch::checkAllContiguous(checked_from,
+                            {logits_arg, targets_arg, logit_lengths_arg, target_lengths_arg});
+  torch::checkDim(checked_from, logits_arg, 2);
+  torch::checkDim(checked_from, targets_arg, 2);
+  torch::checkDim(checked_from, logit_lengths_arg, 1);
+  torch::checkDim(checked_from, target_lengths_arg, 1);
+  torch::checkSameSize(checked_from, logit_lengths_arg, target_lengths_arg);
+
+  const int64_t N = logit_lengths.size(0);
+  const int64_t rows = logits.size(0);
+  const int64_t V = logits.size(1);
+  const int64_t S = targets.size(1);
+
+  if (logits.device().type() == torch::kCPU) {
+    // Same checks as the reference makes before it dispatches on the device
+    // (transducer-loss.cc:49-71); then refuse: this build has no CPU path.
+    TORCH_CHECK(N > 0, "logit_lengths must not be empty");
+    const int64_t sum_all_TU =
+        (logit_lengths.to(torch::kLong) * (target_lengths.to(torch::kLong) + 1)).sum().item<int64_t>();
+    const int64_t targets_max = targets.numel() ? targets.max().item<int32_t>() : INT32_MIN;
+    const int64_t target_len_max = target_lengths.max().item<int32_t>();
+    check_batch_values(logits, targets, sum_all_TU, targets_max, target_len_max, blank);
+    torch::checkDeviceType(checked_from, {logits, targets, logit_lengths, target_lengths},
+                           torch::kCPU);
+    throw std::runtime_error(
+        "optimized_transducer_amd computes on MI355X (HIP) only and has no CPU "
+        "implementation; move logits, targets, logit_lengths and target_lengths "
+        "to a HIP device (tensor.cuda()).");
+  }
+
+  torch::checkAllSameGPU(checked_from,
+                         {logits_arg, targets_arg, logit_lengths_arg, target_lengths_arg});
+  TORCH_CHECK(N > 0, "logit_lengths must not be empty");
+  TORCH_CHECK(targets.size(0) == N, "targets.size(0) is ", targets.size(0),
+              " but there are ", N, " utterances");
+  TORCH_CHECK(rows > 0 && V > 0, "logits must not be empty");
+  TORCH_CHECK(rows <= INT32_MAX && N < INT32_MAX && V <= INT32_MAX && S < OT_MAX_U1 * 64,
+              "tensor sizes exceed what 32-bit row offsets can address");
+
+  c10::hip::HIPGuard device_guard(logits.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+
+  // workspace: status | row_splits | scores_beta | den | lp | alpha | beta
+  const size_t off_splits = align256(sizeof(ot_batch_status));
+  const size_t off_sbeta = off_splits + align256((N + 1) * sizeof(int32_t));
+  const size_t off_den = off_sbeta + align256(N * sizeof(float));
+  const size_t off_lp = off_den + align256(rows * sizeof(float));
+  const size_t off_alpha = off_lp + align256(rows * 2 * sizeof(float));
+  const size_t off_beta = off_alpha + align256(rows * sizeof(float));
+  const size_t total = off_beta + align256(rows * sizeof(float));
+  torch::Tensor workspace =
+      torch::empty({(int64_t)total}, logits.options().dtype(torch::kUInt8));
+  char *w = static_cast<char *>(workspace.data_ptr());
+  auto *status_dev = reinterpret_cast<ot_batch_status *>(w);
+  auto *row_splits = reinterpret_cast<int32_t *>(w + off_splits);
+  auto *scores_beta = reinterpret_cast<float *>(w + off_sbeta);
+  auto *den = reinterpret_cast<float *>(w + off_den);
+  auto *lp = reinterpret_cast<float *>(w + off_lp);
+  auto *alpha = reinterpret_cast<float *>(w + off_alpha);
+  auto *beta = reinterpret_cast<float *>(w + off_beta);
+
+  const float *p_logits = logits.data_ptr<float>();
+  const int32_t *p_targets = S > 0 ? targets.data_ptr<int32_t>() : nullptr;
+  const int32_t *p_T = logit_lengths.data_ptr<int32_t>();
+  const int32_t *p_U = target_lengths.data_ptr<int32_t>();
+
+  // One device pass gathers every fact the checks need; one small D2H copy and
+  // one event wait replace the reference's blocking .item() calls.
+  torch::Tensor status_host = torch::empty(
+      {(int64_t)sizeof(ot_batch_status)},
+      torch::TensorOptions().dtype(torch::kUInt8).device(torch::kCPU).pinned_memory(true));
+  {
+    ScopedTimer timer("prepare", stream);
+    OT_CHECK(ot_row_splits(p_T, p_U, p_targets, (int32_t)N, (int32_t)S, row_splits, status_dev,
+                           stream));
+  }
+  OT_CHECK_HIP(hipMemcpyAsync(status_host.data_ptr(), status_dev, sizeof(ot_batch_status),
+                              hipMemcpyDeviceToHost, stream));
+  hipEvent_t status_ready;
+  OT_CHECK_HIP(hipEventCreateWithFlags(&status_ready, hipEventDisableTiming));
+  OT_CHECK_HIP(hipEventRecord(status_ready, stream));
+
+  // The first streaming kernel only reads and guards every index it derives
+  // from device data, so it can run while the host waits for the facts.
+  const bool blank_ok = (0 <= blank && blank < V);
+  if (blank_ok) {
+    ScopedTimer timer(from_log_softmax ? "gather" : "lse_gather", stream);
+    OT_CHECK(ot_log_probs(p_logits, p_targets, p_U, row_splits, (int32_t)N, (int32_t)S, rows,
+                          (int32_t)V, blank, from_log_softmax, den, lp, stream));
+  }
+  hipError_t ev = hipEventSynchronize(status_ready);
+  (void)hipEventDestroy(status_ready);
+  OT_CHECK_HIP(ev);
+  const ot_batch_status st = *reinterpret_cast<const ot_batch_status *>(status_host.data_ptr());
+
+  check_batch_values(logits, targets, st.sum_tu, S > 0 ? (int64_t)st.targets_max : INT32_MIN,
+                     st.target_len_max, blank);
+  // beyond the reference (which has undefined behaviour for these)
+  TORCH_CHECK(S == 0 || st.targets_min >= 0, "targets.min() is ", st.targets_min,
+              ". Expect targets.min() >= 0");
+  TORCH_CHECK(st.logit_len_min >= 1 && st.target_len_min >= 0,
+              "Expect logit_lengths >= 1 and target_lengths >= 0, but the minima are ",
+              st.logit_len_min, " and ", st.target_len_min);
+  const int32_t max_u1 = st.target_len_max + 1;
+  TORCH_CHECK(max_u1 <= OT_MAX_U1, "target_lengths.max() + 1 is ", max_u1,
+              ", which exceeds the supported ", OT_MAX_U1);
+
+  torch::Tensor scores = torch::empty({N}, logits.options());
+  {
+    ScopedTimer timer("alpha_beta", stream);
+    OT_CHECK(ot_alpha_beta(lp, p_T, p_U, row_splits, (int32_t)N, max_u1, one_sym_per_frame, alpha,
+                           beta, scores.data_ptr<float>(), scores_beta, stream));
+  }
+
+  torch::Tensor gradient;
+  if (logits.requires_grad()) {
+    // cpu.cc:803 / cuda.cu:444: new tensor for log-softmax input;
+    // cpu.cc:814 / cuda.cu:449: the logits buffer itself otherwise.
+    gradient = from_log_softmax ? torch::empty_like(logits) : logits;
+    ScopedTimer timer(from_log_softmax ? "grad_logsoftmax" : "grad_logits", stream);
+    OT_CHECK(ot_gradient(p_logits, lp, den, alpha, beta, p_targets, p_T, p_U, row_splits,
+                         (int32_t)N, (int32_t)S, rows, (int32_t)V, blank, from_log_softmax,
+                         one_sym_per_frame, (float)grad_scale, gradient.data_ptr<float>(),
+                         stream));
+  }
+  if (gradient.defined()) return {scores, gradient};
+  return {scores, torch::nullopt};
+}
+
+// Signature and keyword names of the reference binding
+// (optimized_transducer.cc:14-18).
+std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_transducer_loss(
+    torch::Tensor &logits, const torch::Tensor &targets, const torch::Tensor &logit_lengths,
+    const torch::Tensor &target_lengths, int32_t blank, bool from_log_softmax,
+    bool one_sym_per_frame) {
+  return compute_impl(logits, targets, logit_lengths, target_lengths, blank, from_log_softmax,
+                      one_sym_per_frame, 1.0);
+}
+
+// x *= loss_grad with loss_grad read on the device (no host synchronisation);
+// the kernel returns immediately when loss_grad == 1.
+void scale_by_device_scalar_(torch::Tensor &x, const torch::Tensor &factor) {
+  TORCH_CHECK(x.is_cuda() && factor.is_cuda() && x.device() == factor.device(),
+              "scale_by_device_scalar_: both tensors must be on the same HIP device");
+  TORCH_CHECK(x.scalar_type() == torch::kFloat && factor.scalar_type() == torch::kFloat,
+              "scale_by_device_scalar_: float32 only");
+  TORCH_CHECK(x.is_contiguous() && factor.numel() == 1,
+              "scale_by_device_scalar_: x must be contiguous and factor a single element");
+  c10::hip::HIPGuard device_guard(x.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+  ScopedTimer timer("scale", stream);
+  OT_CHECK(ot_scale_by_device_scalar(x.data_ptr<float>(), x.numel(), factor.data_ptr<float>(),
+                                     stream));
+}
+
+}  // namespace
+
+PYBIND11_MODULE(_optimized_transducer, m) {
+  m.doc() = "MI355X-native transducer loss (drop-in for optimized_transducer's extension module)";
+  m.def("compute_transducer_loss", &compute_transducer_loss, py::arg("logits"),
+        py::arg("targets"), py::arg("logit_lengths"), py::arg("target_lengths"),
+        py::arg("blank"), py::arg("from_log_softmax"), py::arg("one_sym_per_frame"));
+  m.def("compute_transducer_loss_scaled", &compute_impl, py::arg("logits"), py::arg("targets"),
+        py::arg("logit_lengths"), py::arg("target_lengths"), py::arg("blank"),
+        py::arg("from_log_softmax"), py::arg("one_sym_per_frame"), py::arg("grad_scale"),
+        "Same as compute_transducer_loss with the gradient multiplied by grad_scale in the "
+        "gradient kernel (folds the `grad /= N` of reduction='mean').");
+  m.def("scale_by_device_scalar_", &scale_by_device_scalar_, py::arg("x"), py::arg("factor"));
+  m.def("set_profiling", &set_profiling, py::arg("on"));
+  m.def("take_profile", &take_profile);
+}

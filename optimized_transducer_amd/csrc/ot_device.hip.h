@@ -1,0 +1,168 @@
+// Device-side building blocks shared by the transducer-loss kernels (gfx950).
+//
+// Everything here is wave64 code: cross-lane traffic uses DPP controls of the
+// GFX9 family (quad_perm, row_mirror, wave_shr/wave_shl) and falls back to the
+// LDS crossbar (ds_bpermute via __shfl_xor) only for the two widest butterfly
+// steps.
+#ifndef OT_DEVICE_HIP_H_
+#define OT_DEVICE_HIP_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ot {
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;           // streaming kernels: 4 waves per workgroup
+constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kMaxRowsPerBlock = 256; // bounds the utterance table kept in LDS
+
+#define OT_NEG_INF (-__builtin_huge_valf())
+
+// logf(FLT_EPSILON): below this difference the smaller term of a two-term
+// log-add is dropped (reference optimized_transducer/csrc/cpu.cc:15-16,30-34).
+constexpr float kMinLogDiff = -15.9423847198486328125f;
+
+// DPP control words (GFX9 encoding).
+constexpr int kDppQuadXor1 = 0xB1;       // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;       // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141; // lane i <-> 7-i inside 8 lanes
+constexpr int kDppRowMirror = 0x140;     // lane i <-> 15-i inside 16 lanes
+constexpr int kDppWaveShl1 = 0x130;      // lane i reads lane i+1
+constexpr int kDppWaveShr1 = 0x138;      // lane i reads lane i-1
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+
+// Lane i receives x of lane i-1; lane 0 (which has no source) receives fill.
+__device__ __forceinline__ float wave_shift_up(float x, float fill) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, fill),
+                                         __builtin_bit_cast(int, x), kDppWaveShr1,
+                                         0xf, 0xf, false));
+}
+
+// Lane i receives x of lane i+1; lane 63 receives fill.
+__device__ __forceinline__ float wave_shift_down(float x, float fill) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, fill),
+                                         __builtin_bit_cast(int, x), kDppWaveShl1,
+                                         0xf, 0xf, false));
+}
+
+struct MaxOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+struct SumOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+
+// All-reduce over aligned groups of L consecutive lanes (L = 1..64, power of
+// two).  Butterfly: after step s every lane holds the reduction of its aligned
+// 2^s group, so all lanes of a group end with the same bits.
+template <int L, class Op>
+__device__ __forceinline__ float group_allreduce(float v, Op op) {
+  if (L >= 2) v = op(v, dpp_mov<kDppQuadXor1>(v));
+  if (L >= 4) v = op(v, dpp_mov<kDppQuadXor2>(v));
+  if (L >= 8) v = op(v, dpp_mov<kDppRowHalfMirror>(v));
+  if (L >= 16) v = op(v, dpp_mov<kDppRowMirror>(v));
+  if (L >= 32) v = op(v, __shfl_xor(v, 16, kWave));
+  if (L >= 64) v = op(v, __shfl_xor(v, 32, kWave));
+  return v;
+}
+
+// log(exp(a) + exp(b)) exactly as the reference's CPU LogSumExp orders it
+// (cpu.cc:18-35): larger + log1p(exp(smaller - larger)), or just the larger
+// one when the difference is below kMinLogDiff or is NaN (-inf minus -inf).
+__device__ __forceinline__ float log_add(float a, float b) {
+  const float hi = (a < b) ? b : a;
+  const float diff = (a < b) ? (a - b) : (b - a);
+  if (diff >= kMinLogDiff) return hi + log1pf(expf(diff));
+  return hi;
+}
+
+// Largest b in [0, n-1] with splits[b] <= row (splits ascending, splits[0]=0).
+__device__ __forceinline__ int find_utterance(const int32_t *splits, int n, int64_t row) {
+  int lo = 0, hi = n;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if ((int64_t)splits[mid] <= row) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// Utterance table of one workgroup of a per-row streaming kernel.  A workgroup
+// owns a contiguous span of at most kMaxRowsPerBlock rows, which can touch at
+// most that many + 1 utterances (every utterance has at least one row), so the
+// slice of row_splits it needs always fits this fixed LDS footprint.
+struct BlockUtterances {
+  int32_t splits[kMaxRowsPerBlock + 2];
+  int32_t b_lo;
+  int32_t count;  // utterances touched
+
+  // Collective over the workgroup; row_first <= row_last are the block's rows.
+  __device__ __forceinline__ void load(const int32_t *__restrict__ row_splits, int N,
+                                       int64_t row_first, int64_t row_last) {
+    if (threadIdx.x == 0) {
+      const int lo = find_utterance(row_splits, N, row_first);
+      const int hi = find_utterance(row_splits, N, row_last);
+      b_lo = lo;
+      count = hi - lo + 1;
+    }
+    __syncthreads();
+    const int n = count + 1;
+    for (int i = threadIdx.x; i < n && i < kMaxRowsPerBlock + 2; i += blockDim.x)
+      splits[i] = row_splits[b_lo + i];
+    __syncthreads();
+  }
+
+  // Utterance of a row inside the block's span.
+  __device__ __forceinline__ int utterance_of(int64_t row) const {
+    return b_lo + find_utterance(splits, count, row);
+  }
+  __device__ __forceinline__ int32_t split(int b) const { return splits[b - b_lo]; }
+};
+
+// Where a packed row sits in its utterance's lattice.
+struct Cell {
+  int b, t, u, T, U;
+  int64_t row0;  // first row of the utterance
+};
+
+__device__ __forceinline__ Cell decode_row(const BlockUtterances &bu, int64_t row,
+                                           const int32_t *__restrict__ logit_lengths,
+                                           const int32_t *__restrict__ target_lengths) {
+  Cell c;
+  c.b = bu.utterance_of(row);
+  c.row0 = bu.split(c.b);
+  c.U = target_lengths[c.b];
+  c.T = logit_lengths ? logit_lengths[c.b] : 0;
+  const int u1 = c.U + 1 > 0 ? c.U + 1 : 1;
+  const int idx = (int)(row - c.row0);
+  c.t = idx / u1;
+  c.u = idx - c.t * u1;
+  return c;
+}
+
+template <int VEC> struct Vec;
+template <> struct Vec<4> {
+  float v[4];
+  __device__ __forceinline__ void load(const float *p) {
+    const float4 x = *reinterpret_cast<const float4 *>(p);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  }
+  __device__ __forceinline__ void store(float *p) const {
+    *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <> struct Vec<1> {
+  float v[1];
+  __device__ __forceinline__ void load(const float *p) { v[0] = *p; }
+  __device__ __forceinline__ void store(float *p) const { *p = v[0]; }
+};
+
+}  // namespace ot
+#endif  // OT_DEVICE_HIP_H_

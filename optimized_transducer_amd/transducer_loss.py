@@ -1,0 +1,161 @@
+"""Python entry points, mirroring
+optimized_transducer/python/optimized_transducer/transducer_loss.py.
+
+Differences from the reference that do not change results:
+
+* the ``grad /= N`` pass of ``reduction="mean"`` (transducer_loss.py:150) is
+  folded into the gradient kernel as a multiplication by ``1/N``;
+* ``backward`` multiplies by ``loss_grad`` with a kernel that reads the factor
+  on the device and does nothing when it equals 1 (transducer_loss.py:162 always
+  makes a full pass);
+* ``TransducerLoss.__init__`` calls ``super().__init__()`` so the module can
+  actually be called (the reference's class omits it, transducer_loss.py:173-188).
+"""
+import torch
+
+from . import _optimized_transducer
+
+
+class TransducerLossFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(
+        ctx,
+        logits: torch.Tensor,
+        targets: torch.Tensor,
+        logit_lengths: torch.Tensor,
+        target_lengths: torch.Tensor,
+        blank: int,
+        from_log_softmax: bool,
+        one_sym_per_frame: bool,
+        reduction: str = "mean",
+    ) -> torch.Tensor:
+        """See :func:`transducer_loss` for the arguments.
+
+        Caution: when ``from_log_softmax`` is False and ``logits`` requires
+        grad, ``logits`` is overwritten with its gradient (reference
+        transducer_loss.py:45-48).
+        """
+        assert reduction in ("mean", "sum")
+
+        batch_size = logit_lengths.size(0)
+        grad_scale = 1.0 / batch_size if (reduction == "mean" and batch_size > 0) else 1.0
+
+        scores, grad = _optimized_transducer.compute_transducer_loss_scaled(
+            logits=logits,
+            targets=targets,
+            logit_lengths=logit_lengths,
+            target_lengths=target_lengths,
+            blank=blank,
+            from_log_softmax=from_log_softmax,
+            one_sym_per_frame=one_sym_per_frame,
+            grad_scale=grad_scale,
+        )
+
+        loss = -1 * scores
+        if reduction == "mean":
+            loss = loss.mean()
+        elif reduction == "sum":
+            loss = loss.sum()
+
+        ctx.grad = grad
+        return loss
+
+    @staticmethod
+    def backward(ctx, loss_grad):
+        assert loss_grad.numel() == 1, loss_grad.numel()
+        grad = ctx.grad
+        if (
+            loss_grad.is_cuda
+            and loss_grad.device == grad.device
+            and loss_grad.dtype == torch.float32
+            and grad.is_contiguous()
+        ):
+            _optimized_transducer.scale_by_device_scalar_(grad, loss_grad.detach().contiguous())
+        else:
+            grad.mul_(loss_grad)
+        return (
+            grad,  # logits
+            None,  # targets
+            None,  # logit_lengths
+            None,  # target_lengths
+            None,  # blank
+            None,  # from_log_softmax
+            None,  # one_sym_per_frame
+            None,  # reduction
+        )
+
+
+class TransducerLoss(torch.nn.Module):
+    def __init__(self, blank: int, reduction: str = "mean"):
+        """
+        Args:
+          blank: ID of the blank symbol.
+          reduction: "mean" (average over the utterances of the batch) or
+            "sum".  "none" is not supported (reference transducer_loss.py:133).
+        """
+        super().__init__()
+        self.blank = blank
+        self.reduction = reduction
+
+    def forward(
+        self,
+        logits: torch.Tensor,
+        targets: torch.Tensor,
+        logit_lengths: torch.Tensor,
+        target_lengths: torch.Tensor,
+        from_log_softmax: bool,
+        one_sym_per_frame: bool = False,
+    ) -> torch.Tensor:
+        """See :func:`transducer_loss`."""
+        return TransducerLossFunction.apply(
+            logits,
+            targets,
+            logit_lengths,
+            target_lengths,
+            self.blank,
+            from_log_softmax,
+            one_sym_per_frame,
+            self.reduction,
+        )
+
+
+def transducer_loss(
+    logits: torch.Tensor,
+    targets: torch.Tensor,
+    logit_lengths: torch.Tensor,
+    target_lengths: torch.Tensor,
+    blank: int,
+    from_log_softmax: bool,
+    one_sym_per_frame: bool = False,
+    reduction: str = "mean",
+) -> torch.Tensor:
+    """Transducer loss of a packed batch.
+
+    Args:
+      logits: (sum_i T_i * (U_i + 1), V) float32, contiguous, on a HIP device:
+        utterance i's (T_i, U_i + 1, V) joiner output reshaped to 2-D, all
+        utterances concatenated, no padding.  Output of ``nn.Linear`` when
+        ``from_log_softmax`` is False (then it is OVERWRITTEN with its gradient
+        if it requires grad), output of ``log_softmax`` otherwise.
+      targets: (N, max_i U_i) int32, not prepended with blank; every entry,
+        padding included, must be in [0, V).
+      logit_lengths: (N,) int32, T_i.
+      target_lengths: (N,) int32, U_i.
+      blank: ID of the blank symbol, 0 <= blank < V.
+      from_log_softmax: whether ``logits`` already went through log-softmax.
+      one_sym_per_frame: modified transducer - every arc, blank or symbol,
+        advances one frame (needs U_i <= T_i - 1).
+      reduction: "mean" or "sum" over the N utterances.
+    Returns:
+      A 0-dim tensor with the reduced negative log-likelihood.
+    """
+    return TransducerLossFunction.apply(
+        logits,
+        targets,
+        logit_lengths,
+        target_lengths,
+        blank,
+        from_log_softmax,
+        one_sym_per_frame,
+        reduction,
+    )

@@ -1,0 +1,179 @@
+"""ctypes/numpy front end of ``liboracle.so`` (TEST INFRASTRUCTURE ONLY).
+
+The C side restates optimized_transducer/csrc/cpu.cc function by function; this
+module only marshals numpy arrays and mirrors the Python-level arithmetic of
+optimized_transducer/python/optimized_transducer/transducer_loss.py:133-170
+(sign flip, reduction, ``grad /= N``, ``grad *= loss_grad``).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_lib = None
+
+
+def build(force=False):
+    """Compile liboracle.so with the Makefile next to this file."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.run(["make", "-C", _HERE, "liboracle.so"] + (["-B"] if force else []),
+                       check=True, stdout=subprocess.DEVNULL)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.ot_oracle_row_splits.restype = ctypes.c_int64
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _i32(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.int32))
+
+
+def row_splits(logit_lengths, target_lengths):
+    """int32 (N+1,) exclusive prefix of T*(U+1) and the int64 total."""
+    T, U = _i32(logit_lengths), _i32(target_lengths)
+    out = np.empty(T.size + 1, dtype=np.int32)
+    total = lib().ot_oracle_row_splits(_p(T), _p(U), ctypes.c_int32(T.size), _p(out))
+    return out, int(total)
+
+
+def row_ids(splits):
+    splits = _i32(splits)
+    out = np.empty(int(splits[-1]), dtype=np.int32)
+    lib().ot_oracle_row_ids(_p(splits), ctypes.c_int32(splits.size - 1), _p(out))
+    return out
+
+
+def decode_rows(splits, ids, targets, target_lengths):
+    splits, ids, targets, U = _i32(splits), _i32(ids), _i32(targets), _i32(target_lengths)
+    out = np.empty((ids.size, 4), dtype=np.int32)
+    lib().ot_oracle_decode_rows(_p(splits), _p(ids), _p(targets),
+                                ctypes.c_int32(targets.shape[1]), _p(U),
+                                ctypes.c_int32(ids.size), _p(out))
+    return out
+
+
+def _real(dtype):
+    dtype = np.dtype(dtype)
+    assert dtype in (np.float32, np.float64)
+    return dtype, ("_f32" if dtype == np.float32 else "_f64")
+
+
+def logsumexp(logits, dtype=np.float32):
+    dtype, sfx = _real(dtype)
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    den = np.empty(logits.shape[0], dtype=dtype)
+    getattr(lib(), "ot_oracle_logsumexp" + sfx)(
+        _p(logits), ctypes.c_int64(logits.shape[0]), ctypes.c_int32(logits.shape[1]), _p(den))
+    return den
+
+
+def log_probs(logits, den, targets, logit_lengths, target_lengths, blank, dtype=np.float32):
+    dtype, sfx = _real(dtype)
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    targets, T, U = _i32(targets), _i32(logit_lengths), _i32(target_lengths)
+    if den is not None:
+        den = np.ascontiguousarray(den, dtype=dtype)
+    lp = np.empty((logits.shape[0], 2), dtype=dtype)
+    getattr(lib(), "ot_oracle_log_probs" + sfx)(
+        _p(logits), _p(den), _p(targets), ctypes.c_int32(targets.shape[1]), _p(T), _p(U),
+        ctypes.c_int32(T.size), ctypes.c_int32(logits.shape[1]), ctypes.c_int32(blank), _p(lp))
+    return lp
+
+
+def _dp(name, lp, logit_lengths, target_lengths, one_sym_per_frame):
+    dtype, sfx = _real(lp.dtype)
+    lp = np.ascontiguousarray(lp)
+    T, U = _i32(logit_lengths), _i32(target_lengths)
+    out = np.empty(lp.shape[0], dtype=dtype)
+    scores = np.empty(T.size, dtype=dtype)
+    getattr(lib(), name + sfx)(_p(lp), _p(T), _p(U), ctypes.c_int32(T.size),
+                               ctypes.c_int32(int(one_sym_per_frame)), _p(out), _p(scores))
+    return out, scores
+
+
+def alpha(lp, logit_lengths, target_lengths, one_sym_per_frame=False):
+    return _dp("ot_oracle_alpha", lp, logit_lengths, target_lengths, one_sym_per_frame)
+
+
+def beta(lp, logit_lengths, target_lengths, one_sym_per_frame=False):
+    return _dp("ot_oracle_beta", lp, logit_lengths, target_lengths, one_sym_per_frame)
+
+
+def gradient(logits, targets, logit_lengths, target_lengths, blank, den, alpha_, beta_,
+             one_sym_per_frame=False, out=None):
+    dtype, sfx = _real(alpha_.dtype)
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    targets, T, U = _i32(targets), _i32(logit_lengths), _i32(target_lengths)
+    grad = np.empty(logits.shape, dtype=dtype) if out is None else out
+    getattr(lib(), "ot_oracle_gradient" + sfx)(
+        _p(logits), _p(targets), ctypes.c_int32(targets.shape[1]), _p(T), _p(U),
+        ctypes.c_int32(T.size), ctypes.c_int32(logits.shape[1]), ctypes.c_int32(blank),
+        _p(den), _p(alpha_), _p(beta_), ctypes.c_int32(int(one_sym_per_frame)), _p(grad))
+    return grad
+
+
+def compute_transducer_loss(logits, targets, logit_lengths, target_lengths, blank,
+                            from_log_softmax, one_sym_per_frame, want_grad=True,
+                            dtype=np.float32, in_place=False, return_parts=False):
+    """Counterpart of ``_optimized_transducer.compute_transducer_loss``.
+
+    Returns ``(scores, grad)``; scores are +log-likelihoods (cpu.cc:826).  With
+    ``in_place=True`` (float32, logits input) the gradient overwrites ``logits``
+    as the reference does (cpu.cc:814).
+    """
+    dtype, sfx = _real(dtype)
+    assert logits.dtype == np.float32 and logits.flags.c_contiguous
+    targets, T, U = _i32(targets), _i32(logit_lengths), _i32(target_lengths)
+    rows, V = logits.shape
+    work = np.empty(5 * rows, dtype=dtype)
+    scores = np.empty(T.size, dtype=dtype)
+    scores_beta = np.empty(T.size, dtype=dtype)
+    grad = None
+    if want_grad:
+        if in_place and not from_log_softmax and dtype == np.float32:
+            grad = logits
+        else:
+            grad = np.empty((rows, V), dtype=dtype)
+    getattr(lib(), "ot_oracle_transducer_loss" + sfx)(
+        _p(logits), _p(targets), ctypes.c_int32(targets.shape[1]), _p(T), _p(U),
+        ctypes.c_int32(T.size), ctypes.c_int64(rows), ctypes.c_int32(V),
+        ctypes.c_int32(blank), ctypes.c_int32(int(from_log_softmax)),
+        ctypes.c_int32(int(one_sym_per_frame)), _p(work), _p(scores), _p(scores_beta), _p(grad))
+    if return_parts:
+        parts = dict(den=work[:rows], lp=work[rows:3 * rows].reshape(rows, 2),
+                     alpha=work[3 * rows:4 * rows], beta=work[4 * rows:5 * rows],
+                     scores_beta=scores_beta)
+        return scores, grad, parts
+    return scores, grad
+
+
+def transducer_loss(logits, targets, logit_lengths, target_lengths, blank, from_log_softmax,
+                    one_sym_per_frame=False, reduction="mean", loss_grad=1.0,
+                    dtype=np.float32):
+    """Loss value and d(loss * loss_grad)/d(logits), as transducer_loss.py:133-170."""
+    assert reduction in ("mean", "sum")
+    scores, grad = compute_transducer_loss(logits, targets, logit_lengths, target_lengths,
+                                           blank, from_log_softmax, one_sym_per_frame,
+                                           dtype=dtype)
+    real = np.dtype(dtype).type
+    loss = -scores
+    n = len(scores)
+    if reduction == "mean":
+        loss = loss.mean(dtype=dtype)
+        grad /= real(n)
+    else:
+        loss = loss.sum(dtype=dtype)
+    grad *= real(loss_grad)
+    return loss, grad

@@ -1,0 +1,136 @@
+"""ctypes binding of libot_transducer.so for the tests (device pointers come
+from torch tensors; torch is only used for memory and streams here)."""
+import ctypes
+import os
+
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(ROOT, "optimized_transducer_amd", "libot_transducer.so")
+HEADER = os.path.join(ROOT, "include", "ot_transducer.h")
+
+
+class BatchStatus(ctypes.Structure):
+    _fields_ = [("sum_tu", ctypes.c_int64), ("targets_max", ctypes.c_int32),
+                ("targets_min", ctypes.c_int32), ("target_len_max", ctypes.c_int32),
+                ("target_len_min", ctypes.c_int32), ("logit_len_max", ctypes.c_int32),
+                ("logit_len_min", ctypes.c_int32)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.ot_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ot_error_string.restype = ctypes.c_char_p
+    return _lib
+
+
+def ptr(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def check(rc):
+    if rc != 0:
+        raise RuntimeError("ot error %d: %s" % (rc, lib().ot_error_string(rc).decode()))
+
+
+def row_splits(T, U, targets):
+    N = T.numel()
+    splits = torch.empty(N + 1, dtype=torch.int32, device=T.device)
+    status = torch.zeros(ctypes.sizeof(BatchStatus), dtype=torch.uint8, device=T.device)
+    cols = targets.shape[1]
+    check(lib().ot_row_splits(ptr(T), ptr(U), ptr(targets if cols else None), ctypes.c_int32(N),
+                              ctypes.c_int32(cols), ptr(splits), ptr(status), stream()))
+    st = BatchStatus.from_buffer_copy(status.cpu().numpy().tobytes())
+    return splits, st
+
+
+def row_ids(splits, rows):
+    out = torch.empty(rows, dtype=torch.int32, device=splits.device)
+    check(lib().ot_row_ids(ptr(splits), ctypes.c_int32(splits.numel() - 1), ctypes.c_int64(rows),
+                           ptr(out), stream()))
+    return out
+
+
+def log_probs(logits, targets, U, splits, blank, from_log_softmax):
+    rows, V = logits.shape
+    den = None if from_log_softmax else torch.empty(rows, dtype=torch.float32, device=logits.device)
+    lp = torch.full((rows, 2), float("nan"), dtype=torch.float32, device=logits.device)
+    cols = targets.shape[1]
+    check(lib().ot_log_probs(ptr(logits), ptr(targets if cols else None), ptr(U), ptr(splits),
+                             ctypes.c_int32(U.numel()), ctypes.c_int32(cols),
+                             ctypes.c_int64(rows), ctypes.c_int32(V), ctypes.c_int32(blank),
+                             ctypes.c_int32(int(from_log_softmax)), ptr(den), ptr(lp), stream()))
+    return den, lp
+
+
+def alpha_beta(lp, T, U, splits, max_u1, one_sym_per_frame):
+    rows, N = lp.shape[0], T.numel()
+    dev = lp.device
+    alpha = torch.full((rows,), float("nan"), dtype=torch.float32, device=dev)
+    beta = torch.full((rows,), float("nan"), dtype=torch.float32, device=dev)
+    sa = torch.full((N,), float("nan"), dtype=torch.float32, device=dev)
+    sb = torch.full((N,), float("nan"), dtype=torch.float32, device=dev)
+    check(lib().ot_alpha_beta(ptr(lp), ptr(T), ptr(U), ptr(splits), ctypes.c_int32(N),
+                              ctypes.c_int32(max_u1), ctypes.c_int32(int(one_sym_per_frame)),
+                              ptr(alpha), ptr(beta), ptr(sa), ptr(sb), stream()))
+    return alpha, beta, sa, sb
+
+
+def gradient(logits, lp, den, alpha, beta, targets, T, U, splits, blank, from_log_softmax,
+             one_sym_per_frame, grad_scale=1.0, grad=None):
+    rows, V = logits.shape
+    if grad is None:
+        grad = torch.full((rows, V), float("nan"), dtype=torch.float32, device=logits.device)
+    cols = targets.shape[1]
+    check(lib().ot_gradient(ptr(logits), ptr(lp), ptr(den), ptr(alpha), ptr(beta),
+                            ptr(targets if cols else None), ptr(T), ptr(U), ptr(splits),
+                            ctypes.c_int32(T.numel()), ctypes.c_int32(cols), ctypes.c_int64(rows),
+                            ctypes.c_int32(V), ctypes.c_int32(blank),
+                            ctypes.c_int32(int(from_log_softmax)),
+                            ctypes.c_int32(int(one_sym_per_frame)), ctypes.c_float(grad_scale),
+                            ptr(grad), stream()))
+    return grad
+
+
+def transducer_loss(logits, targets, T, U, blank, from_log_softmax, one_sym_per_frame, max_u1,
+                    grad_scale=1.0, grad="new"):
+    """Whole path through ot_transducer_loss.  grad: "new", "inplace" or None."""
+    rows, V = logits.shape
+    N = T.numel()
+    dev = logits.device
+    nbytes = lib().ot_workspace_bytes(ctypes.c_int32(N), ctypes.c_int64(rows))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    scores = torch.full((N,), float("nan"), dtype=torch.float32, device=dev)
+    status = torch.zeros(ctypes.sizeof(BatchStatus), dtype=torch.uint8, device=dev)
+    if grad == "new":
+        g = torch.full((rows, V), float("nan"), dtype=torch.float32, device=dev)
+    elif grad == "inplace":
+        g = logits
+    else:
+        g = None
+    cols = targets.shape[1]
+    check(lib().ot_transducer_loss(
+        ptr(logits), ptr(targets if cols else None), ptr(T), ptr(U), ctypes.c_int32(N),
+        ctypes.c_int32(cols), ctypes.c_int64(rows), ctypes.c_int32(V), ctypes.c_int32(blank),
+        ctypes.c_int32(int(from_log_softmax)), ctypes.c_int32(int(one_sym_per_frame)),
+        ctypes.c_int32(max_u1), ctypes.c_float(grad_scale), ptr(ws), ctypes.c_size_t(nbytes),
+        ptr(scores), ptr(g), ptr(status), stream()))
+    st = BatchStatus.from_buffer_copy(status.cpu().numpy().tobytes())
+    return scores, g, st
+
+
+def scale_by_device_scalar(x, factor):
+    check(lib().ot_scale_by_device_scalar(ptr(x), ctypes.c_int64(x.numel()), ptr(factor), stream()))
+
+
+def copy_floats(src, dst):
+    check(lib().ot_copy_floats(ptr(src), ptr(dst), ctypes.c_int64(src.numel()), stream()))
