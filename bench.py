@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Throughput of the transducer loss (forward + backward) on one MI355X.
+
+A step is ``loss = transducer_loss(logits, ...); loss.backward()`` on one batch
+of synthetic packed logits that are already resident in HBM.  The logits path
+overwrites its input, so every step gets its own pristine copy, cloned before
+the timed region (288 GB of HBM hold dozens of 1.4 GB batches).
+
+Prints ONE JSON line: utterances/s for the whole job, the HBM roofline of the
+dominant kernel (the in-place gradient kernel) measured with hipEvents on the
+launch stream, and the reference's CPU path timed on this machine's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+
+def make_workload(name):
+    import workloads
+    if name == "asr":  # N=32, T~U{200..500}, U~U{20..100}, V=500, logits, sum
+        return workloads.asr_batch()
+    if name == "asr_logsoftmax_modified":
+        return workloads.asr_batch_logsoftmax_modified()
+    if name == "largevocab":
+        return workloads.large_vocab()
+    if name == "ragged":
+        return workloads.ragged()
+    if name == "ragged_modified":
+        return workloads.ragged(one_sym_per_frame=True)
+    if name == "tiny":
+        return workloads.tiny()
+    raise SystemExit("unknown workload %r" % name)
+
+
+def algorithmic_bytes(w):
+    """Bytes per launch each kernel has to move, per packed row of V floats."""
+    R, V = w.rows, w.V
+    if w.from_log_softmax:
+        return {"gather": 16 * R, "alpha_beta": 24 * R, "grad_logsoftmax": (4 * V + 24) * R}
+    return {"lse_gather": (4 * V + 4 + 8) * R, "alpha_beta": 24 * R,
+            "grad_logits": (8 * V + 20) * R}
+
+
+def cpu_baseline(w, logits_host, max_seconds=30.0):
+    """The reference's CPU path (oracle/_ref) or, failing that, the C port, on
+    the same batch; bounded to about max_seconds of CPU time."""
+    import numpy as np
+    import torch
+    from oracle import oracle, ref_loader
+
+    ref = ref_loader.load()
+    threads = torch.get_num_threads()
+    tg = torch.from_numpy(w.targets)
+    T = torch.from_numpy(w.logit_lengths)
+    U = torch.from_numpy(w.target_lengths)
+
+    def once():
+        x = logits_host.clone()
+        t0 = time.perf_counter()
+        if ref is not None:
+            x.requires_grad_(True)
+            scores, grad = ref.compute_transducer_loss(
+                logits=x, targets=tg, logit_lengths=T, target_lengths=U, blank=w.blank,
+                from_log_softmax=w.from_log_softmax, one_sym_per_frame=w.one_sym_per_frame)
+            with torch.no_grad():  # what the reference's autograd.Function does around the call
+                loss = -scores
+                loss = loss.mean() if w.reduction == "mean" else loss.sum()
+                if w.reduction == "mean":
+                    grad /= w.N
+                grad.mul_(torch.ones(()))  # backward's mul_(loss_grad)
+        else:
+            oracle.transducer_loss(x.numpy(), w.targets, w.logit_lengths, w.target_lengths,
+                                   w.blank, w.from_log_softmax, w.one_sym_per_frame, w.reduction)
+        return time.perf_counter() - t0
+
+    times = [once()]
+    while len(times) < 3 and sum(times) + times[-1] < max_seconds:
+        times.append(once())
+    best = float(np.median(times))
+    kind = "reference" if ref is not None else "port"
+    return {
+        "value": w.N / best, "unit": "utterances/s", "cores": threads if ref is not None else 1,
+        "kind": kind,
+        "sample": "%d full batch(es) of workload %s (N=%d, rows=%d, V=%d), median of %d; "
+                  "%s" % (len(times), w.name, w.N, w.rows, w.V, len(times),
+                          "ATen logsumexp on %d threads, lattice and gradient loops single-threaded "
+                          "as the reference runs them" % threads if ref is not None
+                          else "single-threaded C port of the reference's CPU path"),
+        "seconds_per_batch": best,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="asr")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-roofline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build measures one GPU only (got --gpus %d); "
+                         "utterances are independent, so N GPUs shard the batch by utterance "
+                         "and nothing here would change per GPU." % args.gpus)
+
+    import torch
+    import optimized_transducer_amd as ot
+    from optimized_transducer_amd import _optimized_transducer as ext
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda", 0)
+    w = make_workload(args.workload)
+    K, W = args.steps, args.warmup
+
+    pristine = w.logits_torch(dev)
+    targets = torch.from_numpy(w.targets).to(dev)
+    T = torch.from_numpy(w.logit_lengths).to(dev)
+    U = torch.from_numpy(w.target_lengths).to(dev)
+
+    def step(buf):
+        buf.requires_grad_(True)
+        loss = ot.transducer_loss(buf, targets, T, U, w.blank, w.from_log_softmax,
+                                  w.one_sym_per_frame, w.reduction)
+        loss.backward()
+        return loss
+
+    for _ in range(W):
+        step(pristine.clone())
+    torch.cuda.synchronize()
+
+    bufs = [pristine.clone() for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for b in bufs:
+        step(b)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    del bufs
+
+    out = {
+        "metric": "utterances/sec fwd+bwd loss at N=32,V=500 fp32; achieved HBM GB/s vs peak",
+        "value": w.N * K / elapsed, "unit": "utterances/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": 1e3 * elapsed / K, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": w.name, "N": w.N, "V": w.V, "packed_rows": w.rows,
+                   "from_log_softmax": w.from_log_softmax,
+                   "one_sym_per_frame": w.one_sym_per_frame, "reduction": w.reduction,
+                   "logits_bytes": 4 * w.rows * w.V, "seed": w.seed},
+    }
+
+    if not args.no_roofline:
+        # second pass, per-kernel hipEvent timing on the launch stream
+        bufs = [pristine.clone() for _ in range(K)]
+        torch.cuda.synchronize()
+        ext.set_profiling(True)
+        for b in bufs:
+            step(b)
+        torch.cuda.synchronize()
+        ext.set_profiling(False)
+        del bufs
+        per = {}
+        for name, ms in ext.take_profile():
+            per.setdefault(name, []).append(ms)
+        alg = algorithmic_bytes(w)
+        kernels = {}
+        for name, ms in per.items():
+            avg = sum(ms) / len(ms)
+            kernels[name] = {"avg_ms": avg, "launches": len(ms)}
+            if name in alg and avg > 0:
+                kernels[name]["algorithmic_bytes"] = alg[name]
+                kernels[name]["achieved_GBps"] = alg[name] / (avg * 1e-3) / 1e9
+        dom = "grad_logsoftmax" if w.from_log_softmax else "grad_logits"
+        achieved = kernels[dom]["achieved_GBps"]
+        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": achieved,
+                           "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                           "avg_launch_ms": kernels[dom]["avg_ms"],
+                           "algorithmic_bytes_per_launch": alg[dom]}
+        out["kernels"] = kernels
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w, pristine.cpu())
+        out["speedup_vs_cpu"] = out["value"] / out["cpu_baseline"]["value"]
+
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

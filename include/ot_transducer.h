@@ -106,14 +106,20 @@ int ot_alpha_beta(const float *lp, const int32_t *logit_lengths,
  *   only lp is read, logits and den may be NULL.
  * An utterance whose beta(0,0) is not finite gets an all-zero gradient
  * (kernels.cu:558-563).  grad_scale = 1 reproduces the reference; 1/N folds
- * the `grad /= N` of reduction="mean" (transducer_loss.py:150). */
+ * the `grad /= N` of reduction="mean" (transducer_loss.py:150).
+ * Two launches: a per-row pass that turns (alpha, beta, den, targets) into six
+ * coefficients per row in `row_scratch`, then one flat pass over (rows, V). */
 int ot_gradient(const float *logits, const float *lp, const float *den,
                 const float *alpha, const float *beta, const int32_t *targets,
                 const int32_t *logit_lengths, const int32_t *target_lengths,
                 const int32_t *row_splits, int32_t N, int32_t targets_cols,
                 int64_t rows, int32_t V, int32_t blank,
                 int32_t from_log_softmax, int32_t one_sym_per_frame,
-                float grad_scale, float *grad, void *stream);
+                float grad_scale, void *row_scratch, float *grad, void *stream);
+
+/* Bytes of 16-byte aligned device scratch ot_gradient needs in `row_scratch`
+ * (per-row coefficients, 24 bytes per packed row). */
+size_t ot_gradient_scratch_bytes(int64_t rows);
 
 /* In-place x *= *factor for n floats, skipped entirely on the device when
  * *factor == 1.  Replaces ctx.grad.mul_(loss_grad) in backward

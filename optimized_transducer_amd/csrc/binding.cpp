@@ -6,8 +6,8 @@
 // and enqueues the C-ABI kernels of include/ot_transducer.h on torch's current
 // HIP stream.  There is no CPU implementation behind it: CPU tensors are
 // checked like the reference checks them and then rejected.
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <hip/hip_runtime_api.h>
 #include <torch/extension.h>
 
@@ -163,22 +163,21 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   TORCH_CHECK(rows <= INT32_MAX && N < INT32_MAX && V <= INT32_MAX && S < OT_MAX_U1 * 64,
               "tensor sizes exceed what 32-bit row offsets can address");
 
-  c10::hip::HIPGuard device_guard(logits.device());
-  hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+  c10::hip::HIPGuardMasqueradingAsCUDA device_guard(logits.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
 
-  // workspace: status | row_splits | scores_beta | den | lp | alpha | beta
-  const size_t off_splits = align256(sizeof(ot_batch_status));
-  const size_t off_sbeta = off_splits + align256((N + 1) * sizeof(int32_t));
+  // workspace: row_splits | scores_beta | den | lp | alpha | beta | row coefficients
+  const size_t off_sbeta = align256((N + 1) * sizeof(int32_t));
   const size_t off_den = off_sbeta + align256(N * sizeof(float));
   const size_t off_lp = off_den + align256(rows * sizeof(float));
   const size_t off_alpha = off_lp + align256(rows * 2 * sizeof(float));
   const size_t off_beta = off_alpha + align256(rows * sizeof(float));
-  const size_t total = off_beta + align256(rows * sizeof(float));
+  const size_t off_coef = off_beta + align256(rows * sizeof(float));
+  const size_t total = off_coef + align256(ot_gradient_scratch_bytes(rows));
   torch::Tensor workspace =
       torch::empty({(int64_t)total}, logits.options().dtype(torch::kUInt8));
   char *w = static_cast<char *>(workspace.data_ptr());
-  auto *status_dev = reinterpret_cast<ot_batch_status *>(w);
-  auto *row_splits = reinterpret_cast<int32_t *>(w + off_splits);
+  auto *row_splits = reinterpret_cast<int32_t *>(w);
   auto *scores_beta = reinterpret_cast<float *>(w + off_sbeta);
   auto *den = reinterpret_cast<float *>(w + off_den);
   auto *lp = reinterpret_cast<float *>(w + off_lp);
@@ -190,18 +189,19 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   const int32_t *p_T = logit_lengths.data_ptr<int32_t>();
   const int32_t *p_U = target_lengths.data_ptr<int32_t>();
 
-  // One device pass gathers every fact the checks need; one small D2H copy and
-  // one event wait replace the reference's blocking .item() calls.
+  // One device pass gathers every fact the checks need and writes them straight
+  // into pinned host memory; one event wait replaces the reference's blocking
+  // .item() calls (transducer-loss.cc:49,53,62 and cuda.cu:166,169,242,245).
   torch::Tensor status_host = torch::empty(
       {(int64_t)sizeof(ot_batch_status)},
       torch::TensorOptions().dtype(torch::kUInt8).device(torch::kCPU).pinned_memory(true));
+  void *status_dev = nullptr;
+  OT_CHECK_HIP(hipHostGetDevicePointer(&status_dev, status_host.data_ptr(), 0));
   {
     ScopedTimer timer("prepare", stream);
-    OT_CHECK(ot_row_splits(p_T, p_U, p_targets, (int32_t)N, (int32_t)S, row_splits, status_dev,
-                           stream));
+    OT_CHECK(ot_row_splits(p_T, p_U, p_targets, (int32_t)N, (int32_t)S, row_splits,
+                           static_cast<ot_batch_status *>(status_dev), stream));
   }
-  OT_CHECK_HIP(hipMemcpyAsync(status_host.data_ptr(), status_dev, sizeof(ot_batch_status),
-                              hipMemcpyDeviceToHost, stream));
   hipEvent_t status_ready;
   OT_CHECK_HIP(hipEventCreateWithFlags(&status_ready, hipEventDisableTiming));
   OT_CHECK_HIP(hipEventRecord(status_ready, stream));
@@ -246,8 +246,8 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
     ScopedTimer timer(from_log_softmax ? "grad_logsoftmax" : "grad_logits", stream);
     OT_CHECK(ot_gradient(p_logits, lp, den, alpha, beta, p_targets, p_T, p_U, row_splits,
                          (int32_t)N, (int32_t)S, rows, (int32_t)V, blank, from_log_softmax,
-                         one_sym_per_frame, (float)grad_scale, gradient.data_ptr<float>(),
-                         stream));
+                         one_sym_per_frame, (float)grad_scale, w + off_coef,
+                         gradient.data_ptr<float>(), stream));
   }
   if (gradient.defined()) return {scores, gradient};
   return {scores, torch::nullopt};
@@ -272,8 +272,8 @@ void scale_by_device_scalar_(torch::Tensor &x, const torch::Tensor &factor) {
               "scale_by_device_scalar_: float32 only");
   TORCH_CHECK(x.is_contiguous() && factor.numel() == 1,
               "scale_by_device_scalar_: x must be contiguous and factor a single element");
-  c10::hip::HIPGuard device_guard(x.device());
-  hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+  c10::hip::HIPGuardMasqueradingAsCUDA device_guard(x.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
   ScopedTimer timer("scale", stream);
   OT_CHECK(ot_scale_by_device_scalar(x.data_ptr<float>(), x.numel(), factor.data_ptr<float>(),
                                      stream));

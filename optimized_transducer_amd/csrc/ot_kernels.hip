@@ -27,66 +27,72 @@ namespace ot {
 // ---------------------------------------------------------------------------
 // prepare: exclusive scan of T*(U+1) and the reductions the argument checks need
 // ---------------------------------------------------------------------------
-constexpr int kPrepThreads = 1024;
+constexpr int kPrepThreads = 256;
 
+// One workgroup.  Wave 0 scans the sizes 64 at a time with lane shuffles; all
+// waves reduce the lengths and the targets.
 __global__ __launch_bounds__(kPrepThreads) void prepare_kernel(
     const int32_t *__restrict__ logit_lengths, const int32_t *__restrict__ target_lengths,
     const int32_t *__restrict__ targets, int N, int targets_cols,
     int32_t *__restrict__ row_splits, ot_batch_status *__restrict__ status) {
-  __shared__ long long s_scan[kPrepThreads];
-  __shared__ long long s_carry;
   __shared__ int s_red[6];
+  __shared__ long long s_total;
   const int tid = threadIdx.x;
   if (tid == 0) {
-    s_carry = 0;
     s_red[0] = INT32_MIN;  // targets max
     s_red[1] = INT32_MAX;  // targets min
     s_red[2] = INT32_MIN;  // U max
     s_red[3] = INT32_MAX;  // U min
     s_red[4] = INT32_MIN;  // T max
     s_red[5] = INT32_MAX;  // T min
-    row_splits[0] = 0;
   }
   __syncthreads();
 
-  int umax = INT32_MIN, umin = INT32_MAX, tmax = INT32_MIN, tmin = INT32_MAX;
-  for (int base = 0; base < N; base += kPrepThreads) {
-    const int i = base + tid;
-    long long sz = 0;
-    if (i < N) {
-      const int T = logit_lengths[i], U = target_lengths[i];
-      sz = (long long)T * ((long long)U + 1);
-      umax = max(umax, U); umin = min(umin, U);
-      tmax = max(tmax, T); tmin = min(tmin, T);
+  if (tid < kWave) {
+    long long carry = 0;
+    for (int base = 0; base < N; base += kWave) {
+      const int i = base + tid;
+      long long v = 0;
+      if (i < N) v = (long long)logit_lengths[i] * ((long long)target_lengths[i] + 1);
+      for (int ofs = 1; ofs < kWave; ofs <<= 1) {
+        const long long o = __shfl_up(v, ofs, kWave);
+        if (tid >= ofs) v += o;
+      }
+      // int32 wrap-around like cumsum(int32) of the reference
+      if (i < N) row_splits[i + 1] = (int32_t)(uint32_t)(unsigned long long)(carry + v);
+      carry += __shfl(v, kWave - 1, kWave);
     }
-    // Hillis-Steele inclusive scan over the chunk
-    s_scan[tid] = sz;
-    __syncthreads();
-    for (int ofs = 1; ofs < kPrepThreads; ofs <<= 1) {
-      const long long add = (tid >= ofs) ? s_scan[tid - ofs] : 0;
-      __syncthreads();
-      s_scan[tid] += add;
-      __syncthreads();
+    if (tid == 0) {
+      row_splits[0] = 0;
+      s_total = carry;
     }
-    const long long incl = s_carry + s_scan[tid];
-    if (i < N) row_splits[i + 1] = (int32_t)(uint32_t)(unsigned long long)incl;  // int32 wrap like cumsum(int32)
-    __syncthreads();
-    if (tid == kPrepThreads - 1) s_carry = incl;
-    __syncthreads();
   }
 
+  int umax = INT32_MIN, umin = INT32_MAX, tmax = INT32_MIN, tmin = INT32_MAX;
+  for (int i = tid; i < N; i += kPrepThreads) {
+    const int T = logit_lengths[i], U = target_lengths[i];
+    umax = max(umax, U); umin = min(umin, U);
+    tmax = max(tmax, T); tmin = min(tmin, T);
+  }
   int gmax = INT32_MIN, gmin = INT32_MAX;
   const long long ntargets = (long long)N * targets_cols;
   for (long long i = tid; i < ntargets; i += kPrepThreads) {
     const int v = targets[i];
     gmax = max(gmax, v); gmin = min(gmin, v);
   }
-  atomicMax(&s_red[0], gmax); atomicMin(&s_red[1], gmin);
-  atomicMax(&s_red[2], umax); atomicMin(&s_red[3], umin);
-  atomicMax(&s_red[4], tmax); atomicMin(&s_red[5], tmin);
+  for (int ofs = kWave / 2; ofs > 0; ofs >>= 1) {
+    gmax = max(gmax, __shfl_xor(gmax, ofs, kWave)); gmin = min(gmin, __shfl_xor(gmin, ofs, kWave));
+    umax = max(umax, __shfl_xor(umax, ofs, kWave)); umin = min(umin, __shfl_xor(umin, ofs, kWave));
+    tmax = max(tmax, __shfl_xor(tmax, ofs, kWave)); tmin = min(tmin, __shfl_xor(tmin, ofs, kWave));
+  }
+  if ((tid & (kWave - 1)) == 0) {
+    atomicMax(&s_red[0], gmax); atomicMin(&s_red[1], gmin);
+    atomicMax(&s_red[2], umax); atomicMin(&s_red[3], umin);
+    atomicMax(&s_red[4], tmax); atomicMin(&s_red[5], tmin);
+  }
   __syncthreads();
   if (tid == 0) {
-    status->sum_tu = s_carry;
+    status->sum_tu = s_total;
     status->targets_max = s_red[0];
     status->targets_min = s_red[1];
     status->target_len_max = s_red[2];
@@ -153,7 +159,7 @@ __global__ __launch_bounds__(kBlock) void lse_gather_kernel(
 #pragma unroll
       for (int k = 0; k < K; ++k) {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc += expf(x[k].v[e] - m);
+        for (int e = 0; e < VEC; ++e) acc += exp_fast(x[k].v[e] - m);
       }
       s = group_allreduce<L>(acc, SumOp());
     } else {
@@ -176,11 +182,11 @@ __global__ __launch_bounds__(kBlock) void lse_gather_kernel(
         }
         const float nm = fmaxf(lm, cm);
         const float ref = __builtin_isinf(nm) ? 0.f : nm;
-        float acc = (ls == 0.f) ? 0.f : ls * expf((__builtin_isinf(lm) ? 0.f : lm) - ref);
+        float acc = (ls == 0.f) ? 0.f : ls * exp_fast((__builtin_isinf(lm) ? 0.f : lm) - ref);
 #pragma unroll
         for (int k = 0; k < K; ++k) {
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) acc += expf(x[k].v[e] - ref);
+          for (int e = 0; e < VEC; ++e) acc += exp_fast(x[k].v[e] - ref);
         }
         ls = acc;
         lm = nm;
@@ -188,7 +194,7 @@ __global__ __launch_bounds__(kBlock) void lse_gather_kernel(
       m = group_allreduce<L>(lm, MaxOp());
       if (__builtin_isinf(m)) m = 0.f;
       const float lref = __builtin_isinf(lm) ? 0.f : lm;
-      const float part = (ls == 0.f) ? 0.f : ls * expf(lref - m);
+      const float part = (ls == 0.f) ? 0.f : ls * exp_fast(lref - m);
       s = group_allreduce<L>(part, SumOp());
     }
     const float d = logf(s) + m;
@@ -235,89 +241,126 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(
 
 // ---------------------------------------------------------------------------
 // alpha / beta lattice DP: one workgroup per (utterance, direction), one thread
-// per u.  Standard lattice: anti-diagonal sweep (T+U steps); one-symbol-per-
-// frame lattice: every arc advances t, so a row sweep (T steps) suffices.
-// A thread keeps what it hands to its two successors in registers; the value
-// for the neighbouring u travels by a DPP wave shift, and between waves through
-// a double-buffered LDS slot (one barrier per step, none for a single wave).
+// per u.
+//
+// Every thread walks its column u with a start delay, t = n - delay(u) for
+// alpha (mirrored in t and u for beta):
+//   standard lattice        delay = u + wave*kLag   (anti-diagonal wavefront)
+//   one symbol per frame    delay = wave*kLag       (all arcs advance t: row sweep)
+// A thread keeps what it hands to its two successors in registers.  Inside a
+// wave the value for the neighbouring u is exactly one step old and travels by
+// a DPP wave shift.  Across a wave boundary it is kLag+1 steps old: the edge
+// lane writes it to an LDS ring every step and the next wave reads it kLag+1
+// steps later, so one barrier per kChunk = kLag steps orders all LDS traffic
+// (none at all for a single wave).  The lp values do not depend on the
+// recursion and are fetched kChunk steps ahead.
 // ---------------------------------------------------------------------------
 constexpr int kMaxDpWaves = OT_MAX_U1 / kWave;
+constexpr int kChunk = 16;  // steps between barriers
+constexpr int kLag = kChunk;
+constexpr int kRing = 64;   // >= 2*kChunk + 2 slots per wave boundary
+
+#ifndef OT_DP_LOG_ADD
+#define OT_DP_LOG_ADD log_add_fast
+#endif
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 template <bool BETA, bool OSF, bool MULTI>
-__device__ __forceinline__ void lattice_sweep(const float2 *__restrict__ lp, int T, int U,
+__device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int T, int U,
                                               int64_t row0, float *__restrict__ out,
-                                              float *__restrict__ score, float (*s_edge)[kMaxDpWaves + 1]) {
+                                              float *__restrict__ score,
+                                              float (*s_ring)[kRing + 1]) {
   const int u = threadIdx.x;
   const int lane = u & (kWave - 1), wave = u / kWave;
-  const int nwaves = blockDim.x / kWave;
   const int U1 = U + 1;
-  const int diff = T - 1 - U;
-  const int nsteps = OSF ? T : T + U;
-  const float2 ninf2 = make_float2(OT_NEG_INF, OT_NEG_INF);
-  const float2 *lpu = lp + row0;
+  const int wlast = U / kWave;  // wave that owns u == U
+  const int nsteps = (OSF ? T : T + U) + (MULTI ? wlast * kLag : 0);
+  const bool column = u < U1;
+  // (unsigned)(t - u) < band  <=>  u <= t && t - u <= T-1-U   (never, if infeasible)
+  const unsigned band = (unsigned)(max(T - 1 - U, -1) + 1);
 
-  // lattice row of this thread at step n
-  auto t_of = [&](int n) -> int {
-    if (BETA) return OSF ? (T - 1 - n) : (T - 1 + U - n - u);
-    return OSF ? n : (n - u);
+  int delay;
+  if (BETA) delay = (OSF ? 0 : U - u) + (MULTI ? (wlast - wave) * kLag : 0);
+  else delay = (OSF ? 0 : u) + (MULTI ? wave * kLag : 0);
+
+  // This utterance's slice as raw buffers: a cell index outside [0, T*U1)
+  // (t < 0, t >= T, or the forced offset of a thread without a column) reads
+  // as 0 and is not written.
+  const unsigned cells = (unsigned)T * (unsigned)U1;
+  const __amdgpu_buffer_rsrc_t lp_buf = make_buffer(lp + 2 * row0, cells * 8u);
+  const __amdgpu_buffer_rsrc_t out_buf = make_buffer(out + row0, cells * 4u);
+  const unsigned oob = column ? 0u : 0x80000000u;
+  const int dt = BETA ? -1 : 1;
+  const int dcell = BETA ? -U1 : U1;
+  int t = BETA ? (T - 1 + delay) : -delay;  // lattice row at step 0
+  int cell = t * U1 + u;
+
+  auto fetch = [&](int c) -> f32x2 {
+    return __builtin_bit_cast(
+        f32x2, __builtin_amdgcn_raw_buffer_load_b64(lp_buf, ((unsigned)c * 8u) | oob, 0, 0));
   };
-  auto fetch = [&](int n) -> float2 {
-    const int t = t_of(n);
-    const bool valid = (u < U1) & (t >= 0) & (t < T);
-    return valid ? lpu[(int64_t)t * U1 + u] : ninf2;
-  };
+
+  // wave whose edge lane feeds this wave, if any
+  const int src_wave = BETA ? wave + 1 : wave - 1;
+  const bool has_src = MULTI && src_wave >= 0 && src_wave <= wlast;
+  const int edge_lane = BETA ? 0 : kWave - 1;
 
   // alpha: own = alpha(t-1,u)+blank(t-1,u), nb = alpha(t,u)+sym(t,u) handed to u+1
   // beta : own = nb = beta of the cell computed in the previous step
-  float own = OT_NEG_INF, nb = OT_NEG_INF;
+  // The lattice's start cell falls out of the recursion from own = 0:
+  //   alpha(0,0) = log_add(0, -inf) = 0,  beta(T-1,U) = log_add(0 + blank, -inf) = blank.
+  float own = (column && u == (BETA ? U : 0)) ? 0.f : OT_NEG_INF;
+  float nb = OT_NEG_INF;
+  float fin = OT_NEG_INF;  // what the sweep hands out as the utterance's score
 
-  auto step = [&](int n, float2 l) {
-    const int t = t_of(n);
-    const bool valid = (u < U1) & (t >= 0) & (t < T);
-    float edge = OT_NEG_INF;
+  // Ring of kChunk prefetched lp values: slot i is consumed at step n+i and
+  // refilled at once for step n+i+kChunk.
+  f32x2 q[kChunk];
+#pragma unroll
+  for (int i = 0; i < kChunk; ++i) q[i] = fetch(cell + i * dcell);
+
+  for (int n = 0; n < nsteps; n += kChunk) {
+    // the kChunk edge values of this chunk were all written before the last
+    // barrier: fetch them with one LDS read, one lane each
+    float ering = OT_NEG_INF;
     if (MULTI) {
-      const int src = BETA ? wave + 1 : wave - 1;
-      if (src >= 0 && src < nwaves) edge = s_edge[(n + 1) & 1][src];
+      const int s = n - 1 - kLag + lane;
+      if (has_src && lane < kChunk && s >= 0) ering = s_ring[src_wave][s & (kRing - 1)];
     }
-    const float in = BETA ? wave_shift_down(nb, edge) : wave_shift_up(nb, edge);
-    float a;
-    if (BETA) {
-      a = log_add(own + l.x, in + l.y);
-      if (t == T - 1 && u == U) a = l.x;
-    } else {
-      a = log_add(own, in);
-      if (n == 0 && u == 0) a = 0.f;
-    }
-    if (OSF && !(u <= t && t - u <= diff)) a = OT_NEG_INF;
-    if (valid) {
-      out[row0 + (int64_t)t * U1 + u] = a;
+#pragma unroll
+    for (int i = 0; i < kChunk; ++i) {
+      const f32x2 l = q[i];
+      q[i] = fetch(cell + kChunk * dcell);
+      const bool valid = column & ((unsigned)t < (unsigned)T);
+      float edge = OT_NEG_INF;
+      if (MULTI)
+        edge = __builtin_bit_cast(
+            float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ering), i));
+      const float in = BETA ? wave_shift_down(nb, edge) : wave_shift_up(nb, edge);
+      float a = BETA ? OT_DP_LOG_ADD(own + l.x, in + l.y) : OT_DP_LOG_ADD(own, in);
+      if (OSF) a = ((unsigned)(t - u) < band) ? a : OT_NEG_INF;
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, a), out_buf,
+                                            ((unsigned)cell * 4u) | oob, 0, 0);
       if (BETA) {
-        own = nb = a;
-        if (t == 0 && u == 0) *score = a;
+        own = nb = valid ? a : OT_NEG_INF;
+        fin = valid ? a : fin;
       } else {
-        own = a + l.x;
-        nb = a + l.y;
-        if (t == T - 1 && u == U) *score = own;
+        own = valid ? a + l.x : OT_NEG_INF;
+        nb = valid ? a + l.y : OT_NEG_INF;
+        fin = valid ? own : fin;
       }
-    } else {
-      own = nb = OT_NEG_INF;
+      if (MULTI) {
+        // the edge lane publishes nb; every other lane writes a dummy slot
+        float *dst = &s_ring[wave][(lane == edge_lane) ? ((n + i) & (kRing - 1)) : kRing];
+        *dst = nb;
+      }
+      t += dt;
+      cell += dcell;
     }
-    if (MULTI) {
-      if (lane == (BETA ? 0 : kWave - 1)) s_edge[n & 1][wave] = nb;
-      __syncthreads();
-    }
-  };
-
-  // lp values are independent of the recursion: keep them four steps ahead
-  float2 q0 = fetch(0), q1 = fetch(1), q2 = fetch(2), q3 = fetch(3);
-  for (int n = 0; n < nsteps; n += 4) {
-    const float2 p0 = fetch(n + 4), p1 = fetch(n + 5), p2 = fetch(n + 6), p3 = fetch(n + 7);
-    step(n, q0);
-    if (n + 1 < nsteps) step(n + 1, q1);
-    if (n + 2 < nsteps) step(n + 2, q2);
-    if (n + 3 < nsteps) step(n + 3, q3);
-    q0 = p0; q1 = p1; q2 = p2; q3 = p3;
+    if (MULTI) __syncthreads();
   }
+  // alpha: alpha(T-1,U) + blank(T-1,U);  beta: beta(0,0)
+  if (column && u == (BETA ? 0 : U)) *score = fin;
 }
 
 template <bool OSF, bool MULTI>
@@ -326,185 +369,156 @@ __global__ __launch_bounds__(OT_MAX_U1) void alpha_beta_kernel(
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
     float *__restrict__ alpha, float *__restrict__ beta, float *__restrict__ scores_alpha,
     float *__restrict__ scores_beta) {
-  __shared__ float s_edge[2][kMaxDpWaves + 1];
+  __shared__ float s_ring[MULTI ? kMaxDpWaves : 1][kRing + 1];
   const int b = blockIdx.x;
   const int T = logit_lengths[b], U = target_lengths[b];
   const int64_t row0 = row_splits[b];
-  if (MULTI) {
-    if (threadIdx.x < 2 * (kMaxDpWaves + 1)) (&s_edge[0][0])[threadIdx.x] = OT_NEG_INF;
-    __syncthreads();
-  }
-  const float2 *lp2 = reinterpret_cast<const float2 *>(lp);
   if (blockIdx.y == 0)
-    lattice_sweep<false, OSF, MULTI>(lp2, T, U, row0, alpha, scores_alpha + b, s_edge);
+    lattice_sweep<false, OSF, MULTI>(lp, T, U, row0, alpha, scores_alpha + b, s_ring);
   else
-    lattice_sweep<true, OSF, MULTI>(lp2, T, U, row0, beta, scores_beta + b, s_edge);
+    lattice_sweep<true, OSF, MULTI>(lp, T, U, row0, beta, scores_beta + b, s_ring);
 }
 
 // ---------------------------------------------------------------------------
-// gradient kernels
+// gradient: a per-row coefficient pass, then one flat streaming pass
 // ---------------------------------------------------------------------------
-// What a row needs besides its V values.  col1/col2 are the (at most two)
-// columns whose entry has a second exponential subtracted; e1/e2 the beta of
-// the lattice node that arc leads to (0 for the final blank, which leaves the
-// lattice).  Branch order of the reference (blank tests before the target
-// test, cpu.cc:514-523) decides which arc wins when a target equals blank.
-struct RowGrad {
-  float c;      // (alpha + loss) - den          [logits input]   or alpha + loss
-  float bt;     // beta(t, u)
-  float e1, e2;
-  int col1, col2;
-  bool zero;    // row outside the band, or the utterance's likelihood is not finite
-};
+// Everything a row's gradient needs besides its V values, 24 bytes per row:
+//   logits input       f = {c, bt, e1, e2}:  grad[v] = exp((x[v] + c) + bt)
+//                      minus exp((x[v] + c) + e1) at column col1 and
+//                      minus exp((x[v] + c) + e2) at column col2,
+//                      with c = (alpha + loss) - den, bt = beta(t, u)
+//   log-softmax input  f = {v1, v2, 0, 0}: grad is v1 at col1, v2 at col2, else 0
+// e1/e2 are the beta of the node the blank / symbol arc leads to (0 for the
+// final blank, which leaves the lattice).  The reference's branch order (blank
+// tests before the target test, cpu.cc:514-523) decides which arc owns the
+// column when a target equals blank.  col1 == kZeroRow marks an all-zero row
+// (outside the one-symbol-per-frame band, or likelihood not finite).
+constexpr int kZeroRow = -2;
+#ifndef OT_GRAD_EXP
+#define OT_GRAD_EXP exp_any
+#endif
 
-__device__ __forceinline__ RowGrad row_grad(const Cell &c, int64_t row, bool osf, int blank,
-                                            const int32_t *__restrict__ targets, int targets_cols,
-                                            const float *__restrict__ alpha,
-                                            const float *__restrict__ beta,
-                                            const float *__restrict__ den) {
-  RowGrad r;
-  const int U1 = c.U + 1, diff = c.T - 1 - c.U;
-  const float loss = -beta[c.row0];
-  const bool inband = !osf || (c.u <= c.t && c.t - c.u <= diff);
-  r.zero = !inband || !(__builtin_fabsf(loss) < __builtin_huge_valf());
-  r.c = 0.f; r.bt = 0.f; r.e1 = 0.f; r.e2 = 0.f; r.col1 = -1; r.col2 = -1;
-  if (r.zero) return r;
-  const float a = alpha[row];
-  r.bt = beta[row];
-  r.c = den ? (a + loss) - den[row] : a + loss;
-  const bool last = (c.t == c.T - 1) && (c.u == c.U);
-  const bool blank_open = osf ? (c.t - c.u < diff) : (c.t < c.T - 1);
-  const bool has_sym = c.u < c.U;
-  int tgt = -1;
-  if (has_sym && c.u < targets_cols) tgt = targets[(int64_t)c.b * targets_cols + c.u];
-  if (last) {
-    r.col1 = blank; r.e1 = 0.f;
-  } else if (blank_open) {
-    r.col1 = blank; r.e1 = beta[row + U1];
-  }
-  if (has_sym && !(r.col1 >= 0 && tgt == blank)) {
-    r.col2 = tgt;
-    r.e2 = osf ? beta[row + U1 + 1] : beta[row + 1];
-  }
-  return r;
-}
-
-template <int VEC, int L, int K>
-__global__ __launch_bounds__(kBlock) void grad_logits_kernel(
-    const float *logits, float *grad, const float *__restrict__ den,
+template <bool FLS>
+__global__ __launch_bounds__(kBlock) void row_coeff_kernel(
+    const float *__restrict__ lp, const float *__restrict__ den,
     const float *__restrict__ alpha, const float *__restrict__ beta,
     const int32_t *__restrict__ targets, const int32_t *__restrict__ logit_lengths,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits, int N,
-    int targets_cols, int64_t rows, int V, int blank, int osf, float scale, int rows_per_block) {
-  constexpr int G = kWave / L;
+    int targets_cols, int64_t rows, int blank, int osf, float scale,
+    float4 *__restrict__ coef_f, int2 *__restrict__ coef_i) {
   __shared__ BlockUtterances bu;
-  const int64_t row_first = (int64_t)blockIdx.x * rows_per_block;
-  const int64_t row_end = min(rows, row_first + rows_per_block);
+  const int64_t row_first = (int64_t)blockIdx.x * kBlock;
+  const int64_t row_end = min(rows, row_first + kBlock);
   bu.load(row_splits, N, row_first, row_end - 1);
-
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int sub = lane % L, g = lane / L;
-  const int nvec = V / VEC;
-
-  for (int64_t base = row_first + (int64_t)wave * G; base < row_end; base += kWavesPerBlock * G) {
-    const int64_t row = base + g;
-    if (row >= row_end) continue;
-    const float *p = logits + row * (int64_t)V;
-    float *q = grad + row * (int64_t)V;
-
-    // issue the row's first chunk of loads before the (dependent) scalar lookups
-    Vec<VEC> x[K];
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-      const int j = k * L + sub;
-      if (j < nvec) x[k].load(p + (int64_t)j * VEC);
-    }
+  const int64_t row = row_first + threadIdx.x;
+  if (row >= row_end) return;
+  float4 f = make_float4(0.f, 0.f, 0.f, 0.f);
+  int2 ci = make_int2(kZeroRow, -1);
+  if (row < (int64_t)row_splits[N]) {
     const Cell c = decode_row(bu, row, logit_lengths, target_lengths);
-    const RowGrad r = row_grad(c, row, osf != 0, blank, targets, targets_cols, alpha, beta, den);
-    const int j1 = r.col1 >= 0 ? r.col1 / VEC : -1, j2 = r.col2 >= 0 ? r.col2 / VEC : -1;
-
-    for (int c0 = 0; c0 < nvec; c0 += L * K) {
-      if (c0 > 0) {
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-          const int j = c0 + k * L + sub;
-          if (j < nvec) x[k].load(p + (int64_t)j * VEC);
-        }
+    const int U1 = c.U + 1, diff = c.T - 1 - c.U;
+    const float loss = -beta[c.row0];
+    const bool inband = !osf || (c.u <= c.t && c.t - c.u <= diff);
+    if (inband && __builtin_fabsf(loss) < __builtin_huge_valf()) {
+      const float a = alpha[row];
+      const float bt = beta[row];
+      const float cc = FLS ? a + loss : (a + loss) - den[row];
+      const bool last = (c.t == c.T - 1) && (c.u == c.U);
+      const bool blank_open = osf ? (c.t - c.u < diff) : (c.t < c.T - 1);
+      const bool has_sym = c.u < c.U;
+      int tgt = -1;
+      if (has_sym && c.u < targets_cols) tgt = targets[(int64_t)c.b * targets_cols + c.u];
+      int col1 = -1, col2 = -1;
+      float e1 = 0.f, e2 = 0.f;
+      if (last) {
+        col1 = blank;
+      } else if (blank_open) {
+        col1 = blank;
+        e1 = beta[row + U1];
       }
-#pragma unroll
-      for (int k = 0; k < K; ++k) {
-        const int j = c0 + k * L + sub;
-        if (j >= nvec) continue;
-        Vec<VEC> y;
-        if (r.zero) {
-#pragma unroll
-          for (int e = 0; e < VEC; ++e) y.v[e] = 0.f;
-        } else {
-#pragma unroll
-          for (int e = 0; e < VEC; ++e) y.v[e] = expf((x[k].v[e] + r.c) + r.bt);
-          if (j == j1 || j == j2) {
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-              const int col = j * VEC + e;
-              if (col == r.col1) y.v[e] -= expf((x[k].v[e] + r.c) + r.e1);
-              if (col == r.col2) y.v[e] -= expf((x[k].v[e] + r.c) + r.e2);
-            }
-          }
-          if (scale != 1.f) {
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) y.v[e] *= scale;
-          }
-        }
-        y.store(q + (int64_t)j * VEC);
+      if (has_sym && !(col1 >= 0 && tgt == blank)) {
+        col2 = tgt;
+        e2 = osf ? beta[row + U1 + 1] : beta[row + 1];
+      }
+      ci = make_int2(col1, col2);
+      if (FLS) {
+        const float2 l = reinterpret_cast<const float2 *>(lp)[row];
+        f.x = col1 >= 0 ? -OT_GRAD_EXP((l.x + cc) + e1) * scale : 0.f;
+        f.y = col2 >= 0 ? -OT_GRAD_EXP((l.y + cc) + e2) * scale : 0.f;
+      } else {
+        f = make_float4(cc, bt, e1, e2);
       }
     }
   }
+  coef_f[row] = f;
+  coef_i[row] = ci;
 }
 
-template <int VEC, int L>
-__global__ __launch_bounds__(kBlock) void grad_logsoftmax_kernel(
-    const float *__restrict__ lp, float *__restrict__ grad, const float *__restrict__ alpha,
-    const float *__restrict__ beta, const int32_t *__restrict__ targets,
-    const int32_t *__restrict__ logit_lengths, const int32_t *__restrict__ target_lengths,
-    const int32_t *__restrict__ row_splits, int N, int targets_cols, int64_t rows, int V,
-    int blank, int osf, float scale, int rows_per_block) {
-  constexpr int G = kWave / L;
-  __shared__ BlockUtterances bu;
-  const int64_t row_first = (int64_t)blockIdx.x * rows_per_block;
-  const int64_t row_end = min(rows, row_first + rows_per_block);
-  bu.load(row_splits, N, row_first, row_end - 1);
+// Flat pass over the (rows, V) array in units of VEC floats: unit i belongs to
+// row i / nvec.  Consecutive lanes touch consecutive 16-byte units, so every
+// wave instruction moves one aligned, contiguous 1 KiB whatever V is; a
+// workgroup owns kGradUnroll * 256 consecutive units and exists only for them
+// (one-shot grid: the measured optimum for a read-modify-write stream here).
+constexpr int kGradUnroll = 4;
 
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int sub = lane % L, g = lane / L;
-  const int nvec = V / VEC;
+template <int VEC, bool FLS>
+__global__ __launch_bounds__(kBlock) void grad_flat_kernel(
+    const float *logits, float *grad, const float4 *__restrict__ coef_f,
+    const int2 *__restrict__ coef_i, int64_t nunits, int nvec, float inv_nvec, float scale) {
+  const int64_t base = (int64_t)blockIdx.x * (kGradUnroll * kBlock);
+  const int64_t row_base = base / nvec;
+  const int rem_base = (int)(base - row_base * nvec);
 
-  for (int64_t base = row_first + (int64_t)wave * G; base < row_end; base += kWavesPerBlock * G) {
-    const int64_t row = base + g;
-    if (row >= row_end) continue;
-    float *q = grad + row * (int64_t)V;
-    const Cell c = decode_row(bu, row, logit_lengths, target_lengths);
-    const RowGrad r = row_grad(c, row, osf != 0, blank, targets, targets_cols, alpha, beta, nullptr);
-    float v1 = 0.f, v2 = 0.f;
-    if (!r.zero) {
-      const float2 l = reinterpret_cast<const float2 *>(lp)[row];
-      if (r.col1 >= 0) v1 = -expf((l.x + r.c) + r.e1) * scale;
-      if (r.col2 >= 0) v2 = -expf((l.y + r.c) + r.e2) * scale;
-    }
-    const int j1 = r.col1 >= 0 ? r.col1 / VEC : -1, j2 = r.col2 >= 0 ? r.col2 / VEC : -1;
-    for (int j = sub; j < nvec; j += L) {
-      Vec<VEC> y;
+  Vec<VEC> x[kGradUnroll];
+  int rows[kGradUnroll], col0[kGradUnroll];
+#pragma unroll
+  for (int k = 0; k < kGradUnroll; ++k) {
+    const int local = k * kBlock + (int)threadIdx.x;
+    if (!FLS && base + local < nunits) x[k].load(logits + (base + local) * VEC);
+    // idx < nvec + 1024 is exact in float; one correction step fixes the quotient
+    const int idx = rem_base + local;
+    int q = (int)((float)idx * inv_nvec);
+    if (q * nvec > idx) --q; else if ((q + 1) * nvec <= idx) ++q;
+    rows[k] = q;
+    col0[k] = (idx - q * nvec) * VEC;
+  }
+#pragma unroll
+  for (int k = 0; k < kGradUnroll; ++k) {
+    const int local = k * kBlock + (int)threadIdx.x;
+    if (base + local >= nunits) continue;
+    const int64_t row = row_base + rows[k];
+    const float4 f = coef_f[row];
+    const int2 ci = coef_i[row];
+    Vec<VEC> y;
+    if (FLS) {
 #pragma unroll
       for (int e = 0; e < VEC; ++e) y.v[e] = 0.f;
-      if (j == j1 || j == j2) {
+      const unsigned d1 = (unsigned)(ci.x - col0[k]), d2 = (unsigned)(ci.y - col0[k]);
+      if (d1 < (unsigned)VEC || d2 < (unsigned)VEC) {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-          const int col = j * VEC + e;
-          if (col == r.col1) y.v[e] = v1;
-          if (col == r.col2) y.v[e] = v2;
+          if (d1 == (unsigned)e) y.v[e] = f.x;
+          if (d2 == (unsigned)e) y.v[e] = f.y;
         }
       }
-      y.store(q + (int64_t)j * VEC);
+    } else {
+      const bool zero = ci.x == kZeroRow;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) y.v[e] = zero ? 0.f : OT_GRAD_EXP((x[k].v[e] + f.x) + f.y);
+      const unsigned d1 = (unsigned)(ci.x - col0[k]), d2 = (unsigned)(ci.y - col0[k]);
+      if (d1 < (unsigned)VEC || d2 < (unsigned)VEC) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          if (d1 == (unsigned)e) y.v[e] -= OT_GRAD_EXP((x[k].v[e] + f.x) + f.z);
+          if (d2 == (unsigned)e) y.v[e] -= OT_GRAD_EXP((x[k].v[e] + f.x) + f.w);
+        }
+      }
+      if (scale != 1.f) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) y.v[e] *= scale;
+      }
     }
+    y.store_stream(grad + (base + local) * VEC);
   }
 }
 
@@ -582,14 +596,6 @@ static inline bool is_aligned16(const void *p) { return (reinterpret_cast<uintpt
 #define OT_DISPATCH(KERNEL, T_, ...)                                       \
   if ((T_).vec == 4) { OT_DISPATCH_L(KERNEL, 4, (T_).L, (T_).K, __VA_ARGS__) } \
   else { OT_DISPATCH_L(KERNEL, 1, (T_).L, (T_).K, __VA_ARGS__) }
-
-#define OT_DISPATCH_L_ONLY(KERNEL, VEC_, L_, ...)                                                   \
-  switch (L_) {                                                                                     \
-    case 8: hipLaunchKernelGGL((KERNEL<VEC_, 8>), grid, dim3(kBlock), 0, s, __VA_ARGS__); break;    \
-    case 16: hipLaunchKernelGGL((KERNEL<VEC_, 16>), grid, dim3(kBlock), 0, s, __VA_ARGS__); break;  \
-    case 32: hipLaunchKernelGGL((KERNEL<VEC_, 32>), grid, dim3(kBlock), 0, s, __VA_ARGS__); break;  \
-    default: hipLaunchKernelGGL((KERNEL<VEC_, 64>), grid, dim3(kBlock), 0, s, __VA_ARGS__); break;  \
-  }
 
 static inline int launch_status() { return (int)hipGetLastError(); }
 
@@ -673,34 +679,54 @@ int ot_gradient(const float *logits, const float *lp, const float *den, const fl
                 const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
                 int32_t targets_cols, int64_t rows, int32_t V, int32_t blank,
                 int32_t from_log_softmax, int32_t one_sym_per_frame, float grad_scale,
-                float *grad, void *stream) {
-  if (!alpha || !beta || !logit_lengths || !target_lengths || !row_splits || !grad || N <= 0 ||
-      rows <= 0 || rows > INT32_MAX || V <= 0 || blank < 0 || blank >= V || targets_cols < 0 ||
-      (targets_cols > 0 && !targets))
+                void *row_scratch, float *grad, void *stream) {
+  if (!alpha || !beta || !logit_lengths || !target_lengths || !row_splits || !grad ||
+      !row_scratch || N <= 0 || rows <= 0 || rows > INT32_MAX || V <= 0 || blank < 0 ||
+      blank >= V || targets_cols < 0 || (targets_cols > 0 && !targets))
     return OT_E_BAD_ARG;
   if (from_log_softmax ? (!lp || grad == logits) : (!logits || !den)) return OT_E_BAD_ARG;
-  if ((reinterpret_cast<uintptr_t>(grad) & 3) || (reinterpret_cast<uintptr_t>(logits) & 3))
+  if ((reinterpret_cast<uintptr_t>(grad) & 3) || (reinterpret_cast<uintptr_t>(logits) & 3) ||
+      (reinterpret_cast<uintptr_t>(row_scratch) & 15))
     return OT_E_MISALIGNED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool aligned = is_aligned16(grad) && (from_log_softmax || is_aligned16(logits));
-  const RowTiling t = pick_tiling(V, aligned);
-  const dim3 grid((unsigned)((rows + t.rows_per_block - 1) / t.rows_per_block));
-  if (from_log_softmax) {
-    if (t.vec == 4) {
-      OT_DISPATCH_L_ONLY(grad_logsoftmax_kernel, 4, t.L, lp, grad, alpha, beta, targets,
-                         logit_lengths, target_lengths, row_splits, N, targets_cols, rows, V,
-                         blank, one_sym_per_frame, grad_scale, t.rows_per_block)
-    } else {
-      OT_DISPATCH_L_ONLY(grad_logsoftmax_kernel, 1, t.L, lp, grad, alpha, beta, targets,
-                         logit_lengths, target_lengths, row_splits, N, targets_cols, rows, V,
-                         blank, one_sym_per_frame, grad_scale, t.rows_per_block)
-    }
-  } else {
-    OT_DISPATCH(grad_logits_kernel, t, logits, grad, den, alpha, beta, targets, logit_lengths,
-                target_lengths, row_splits, N, targets_cols, rows, V, blank, one_sym_per_frame,
-                grad_scale, t.rows_per_block)
+  float4 *coef_f = static_cast<float4 *>(row_scratch);
+  int2 *coef_i = reinterpret_cast<int2 *>(coef_f + rows);
+  {
+    const dim3 grid((unsigned)((rows + kBlock - 1) / kBlock));
+    if (from_log_softmax)
+      hipLaunchKernelGGL(row_coeff_kernel<true>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
+                         targets, logit_lengths, target_lengths, row_splits, N, targets_cols, rows,
+                         blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
+    else
+      hipLaunchKernelGGL(row_coeff_kernel<false>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
+                         targets, logit_lengths, target_lengths, row_splits, N, targets_cols, rows,
+                         blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
+    const int rc = launch_status();
+    if (rc) return rc;
   }
+  const bool aligned = is_aligned16(grad) && (from_log_softmax || is_aligned16(logits));
+  const int vec = (aligned && V % 4 == 0) ? 4 : 1;
+  const int nvec = V / vec;
+  const int64_t nunits = rows * nvec;
+  const int64_t per_block = (int64_t)kGradUnroll * kBlock;
+  const int64_t blocks = (nunits + per_block - 1) / per_block;
+  if (blocks > INT32_MAX) return OT_E_BAD_ARG;
+  const dim3 grid((unsigned)blocks);
+  const float inv_nvec = 1.0f / (float)nvec;
+#define OT_LAUNCH_GRAD(VEC_, FLS_)                                                            \
+  hipLaunchKernelGGL((grad_flat_kernel<VEC_, FLS_>), grid, dim3(kBlock), 0, s, logits, grad,  \
+                     coef_f, coef_i, nunits, nvec, inv_nvec, grad_scale)
+  if (from_log_softmax) {
+    if (vec == 4) OT_LAUNCH_GRAD(4, true); else OT_LAUNCH_GRAD(1, true);
+  } else {
+    if (vec == 4) OT_LAUNCH_GRAD(4, false); else OT_LAUNCH_GRAD(1, false);
+  }
+#undef OT_LAUNCH_GRAD
   return launch_status();
+}
+
+size_t ot_gradient_scratch_bytes(int64_t rows) {
+  return rows > 0 ? (size_t)rows * (sizeof(float4) + sizeof(int2)) : 0;
 }
 
 int ot_scale_by_device_scalar(float *x, int64_t n, const float *factor, void *stream) {
@@ -725,6 +751,7 @@ size_t ot_workspace_bytes(int32_t N, int64_t rows) {
   b += align256((size_t)rows * 2 * sizeof(float));   // lp
   b += align256((size_t)rows * sizeof(float));       // alpha
   b += align256((size_t)rows * sizeof(float));       // beta
+  b += align256(ot_gradient_scratch_bytes(rows));    // per-row gradient coefficients
   return b;
 }
 
@@ -743,7 +770,8 @@ int ot_transducer_loss(const float *logits, const int32_t *targets, const int32_
   float *den = reinterpret_cast<float *>(w);            w += align256((size_t)rows * sizeof(float));
   float *lp = reinterpret_cast<float *>(w);             w += align256((size_t)rows * 2 * sizeof(float));
   float *alpha = reinterpret_cast<float *>(w);          w += align256((size_t)rows * sizeof(float));
-  float *beta = reinterpret_cast<float *>(w);
+  float *beta = reinterpret_cast<float *>(w);           w += align256((size_t)rows * sizeof(float));
+  void *row_scratch = w;
   int rc = ot_row_splits(logit_lengths, target_lengths, targets, N, targets_cols, row_splits,
                          status, stream);
   if (rc) return rc;
@@ -756,7 +784,7 @@ int ot_transducer_loss(const float *logits, const int32_t *targets, const int32_
   if (grad)
     rc = ot_gradient(logits, lp, den, alpha, beta, targets, logit_lengths, target_lengths,
                      row_splits, N, targets_cols, rows, V, blank, from_log_softmax,
-                     one_sym_per_frame, grad_scale, grad, stream);
+                     one_sym_per_frame, grad_scale, row_scratch, grad, stream);
   return rc;
 }
 

@@ -8,6 +8,9 @@ Differences from the reference that do not change results:
 * ``backward`` multiplies by ``loss_grad`` with a kernel that reads the factor
   on the device and does nothing when it equals 1 (transducer_loss.py:162 always
   makes a full pass);
+* ``backward`` returns a fresh alias of the gradient buffer, so that autograd
+  can adopt it as ``logits.grad`` without the (rows, V) copy the reference's
+  shared tensor object forces when ``logits`` is a leaf;
 * ``TransducerLoss.__init__`` calls ``super().__init__()`` so the module can
   actually be called (the reference's class omits it, transducer_loss.py:173-188).
 """
@@ -63,7 +66,11 @@ class TransducerLossFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, loss_grad):
         assert loss_grad.numel() == 1, loss_grad.numel()
-        grad = ctx.grad
+        # Hand autograd a fresh alias of the gradient buffer and drop ours: when
+        # `logits` is a leaf, autograd then adopts the buffer as logits.grad
+        # instead of cloning (rows, V) floats because others still hold it.
+        grad = ctx.grad.detach()
+        ctx.grad = None
         if (
             loss_grad.is_cuda
             and loss_grad.device == grad.device

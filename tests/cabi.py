@@ -6,7 +6,8 @@ import os
 import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIB_PATH = os.path.join(ROOT, "optimized_transducer_amd", "libot_transducer.so")
+LIB_PATH = os.environ.get(
+    "OT_TRANSDUCER_LIB", os.path.join(ROOT, "optimized_transducer_amd", "libot_transducer.so"))
 HEADER = os.path.join(ROOT, "include", "ot_transducer.h")
 
 
@@ -25,6 +26,7 @@ def lib():
     if _lib is None:
         _lib = ctypes.CDLL(LIB_PATH)
         _lib.ot_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ot_gradient_scratch_bytes.restype = ctypes.c_size_t
         _lib.ot_error_string.restype = ctypes.c_char_p
     return _lib
 
@@ -91,13 +93,15 @@ def gradient(logits, lp, den, alpha, beta, targets, T, U, splits, blank, from_lo
     if grad is None:
         grad = torch.full((rows, V), float("nan"), dtype=torch.float32, device=logits.device)
     cols = targets.shape[1]
+    scratch = torch.empty(lib().ot_gradient_scratch_bytes(ctypes.c_int64(rows)), dtype=torch.uint8,
+                          device=logits.device)
     check(lib().ot_gradient(ptr(logits), ptr(lp), ptr(den), ptr(alpha), ptr(beta),
                             ptr(targets if cols else None), ptr(T), ptr(U), ptr(splits),
                             ctypes.c_int32(T.numel()), ctypes.c_int32(cols), ctypes.c_int64(rows),
                             ctypes.c_int32(V), ctypes.c_int32(blank),
                             ctypes.c_int32(int(from_log_softmax)),
                             ctypes.c_int32(int(one_sym_per_frame)), ctypes.c_float(grad_scale),
-                            ptr(grad), stream()))
+                            ptr(scratch), ptr(grad), stream()))
     return grad
 
 
