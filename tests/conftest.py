@@ -1,0 +1,35 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+def _ensure_built():
+    """Load what is built; compile only if nothing is there."""
+    pkg = os.path.join(ROOT, "optimized_transducer_amd")
+    if not (os.path.exists(os.path.join(pkg, "libot_transducer.so"))
+            and os.path.exists(os.path.join(pkg, "_optimized_transducer.so"))):
+        from optimized_transducer_amd import build
+        build.build_all()
+    from oracle import oracle
+    oracle.build()
+
+
+_ensure_built()
+
+
+@pytest.fixture(scope="session")
+def device():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda", 0)

@@ -1,0 +1,267 @@
+"""GPU parity of the whole path: the Python entry points of the package and
+ot_transducer_loss of the C ABI, against the golden vectors of the compiled
+reference, the CPU oracle and - at the benchmark's full sizes - properties that
+do not depend on size plus the oracle run on a slice of the batch."""
+import numpy as np
+import pytest
+import torch
+
+import cabi
+import helpers
+import workloads
+from helpers import ATOL, RTOL
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+MODES = [(False, False), (False, True), (True, False), (True, True)]  # (from_log_softmax, one_sym)
+
+
+def _dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def _run_api(x, tg, T, U, blank, fls, osf, reduction, device, upstream=1.0, module=False):
+    import optimized_transducer_amd as ot
+    logits = _dev(x, device).requires_grad_(True)
+    args = (logits, _dev(tg, device), _dev(T, device), _dev(U, device))
+    if module:
+        loss = ot.TransducerLoss(blank=blank, reduction=reduction)(*args, fls, osf)
+    else:
+        loss = ot.transducer_loss(*args, blank, fls, one_sym_per_frame=osf, reduction=reduction)
+    (loss * upstream if upstream != 1.0 else loss).backward()
+    return loss, logits
+
+
+# ------------------------------------------------------------------ golden vectors
+@pytest.mark.parametrize("path", helpers.golden_files(), ids=lambda p: p.split("/")[-1][:-4])
+def test_golden_vectors_of_the_compiled_reference(path, device):
+    g = np.load(path)
+    T, U, tg, blank = g["logit_lengths"], g["target_lengths"], g["targets"], int(g["blank"])
+    for fls, osf in helpers.golden_modes(g):
+        x = helpers.log_softmax32(g["logits"]) if fls else g["logits"]
+        ws, wg = g["scores_fls%d_osf%d" % (fls, osf)], g["grad_fls%d_osf%d" % (fls, osf)]
+        loss, logits = _run_api(x, tg, T, U, blank, fls, osf, "sum", device)
+        assert np.allclose(loss.item(), -ws.sum(dtype=np.float64), rtol=RTOL, atol=ATOL)
+        got = logits.grad.cpu().numpy()
+        tol = helpers.lattice_noise_tolerance(wg, helpers.per_row(ws, T, U))
+        assert (np.abs(got - wg) <= tol).all(), (fls, osf, np.abs(got - wg).max())
+        if np.abs(ws).max() < 50:  # short lattices: the plain north-star tolerance holds
+            assert np.allclose(got, wg, rtol=RTOL, atol=ATOL)
+
+
+# ------------------------------------------------------------------ Python API
+@pytest.mark.parametrize("reduction", ["mean", "sum"])
+@pytest.mark.parametrize("fls,osf", MODES)
+def test_python_api_matches_oracle(fls, osf, reduction, device):
+    w = workloads.tiny(from_log_softmax=fls, one_sym_per_frame=osf)
+    x = w.logits_numpy()
+    want_loss, want_grad = oracle.transducer_loss(x.copy(), w.targets, w.logit_lengths,
+                                                  w.target_lengths, w.blank, fls, osf, reduction,
+                                                  loss_grad=3.0)
+    loss, logits = _run_api(x, w.targets, w.logit_lengths, w.target_lengths, w.blank, fls, osf,
+                            reduction, device, upstream=3.0)  # as test_compute_transducer_loss.py:92
+    assert loss.dim() == 0 and loss.dtype == torch.float32
+    assert np.allclose(loss.item(), want_loss, rtol=RTOL, atol=ATOL)
+    s, _ = oracle.compute_transducer_loss(x.copy(), w.targets, w.logit_lengths, w.target_lengths,
+                                          w.blank, fls, osf)
+    scale = 3.0 / (w.N if reduction == "mean" else 1)
+    tol = scale * helpers.lattice_noise_tolerance(want_grad / scale,
+                                                  helpers.per_row(s, w.logit_lengths, w.target_lengths))
+    got = logits.grad.cpu().numpy()
+    assert (np.abs(got - want_grad) <= tol).all(), np.abs(got - want_grad).max()
+    # arbiter: the GPU is as close to the float64 evaluation as the fp32 reference arithmetic is
+    _, g64 = oracle.transducer_loss(x.copy(), w.targets, w.logit_lengths, w.target_lengths,
+                                    w.blank, fls, osf, reduction, loss_grad=3.0, dtype=np.float64)
+    assert np.abs(got - g64).max() <= 2 * np.abs(want_grad - g64).max() + 1e-6
+
+
+def test_in_place_and_aliasing_semantics(device):
+    import optimized_transducer_amd as ot
+    w = workloads.tiny()
+    x = w.logits_numpy()
+    tg, T, U = _dev(w.targets, device), _dev(w.logit_lengths, device), _dev(w.target_lengths, device)
+    # logits input + requires_grad: the buffer is overwritten and IS the gradient (cpu.cc:814)
+    logits = _dev(x, device).requires_grad_(True)
+    ptr = logits.data_ptr()
+    loss = ot.transducer_loss(logits, tg, T, U, 0, False, reduction="sum")
+    assert not np.array_equal(logits.detach().cpu().numpy(), x)
+    loss.backward()
+    assert logits.grad.data_ptr() == ptr  # adopted, not cloned
+    assert torch.equal(logits.grad, logits.detach())
+    # no grad wanted: nothing is written
+    logits2 = _dev(x, device)
+    loss2 = ot.transducer_loss(logits2, tg, T, U, 0, False, reduction="sum")
+    assert np.array_equal(logits2.cpu().numpy(), x) and not loss2.requires_grad
+    assert np.allclose(loss2.item(), loss.item(), rtol=1e-6)
+    # log-softmax input: the input survives, the gradient is a new tensor (cpu.cc:803)
+    xl = helpers.log_softmax32(x)
+    logits3 = _dev(xl, device).requires_grad_(True)
+    ot.transducer_loss(logits3, tg, T, U, 0, True, reduction="sum").backward()
+    assert np.array_equal(logits3.detach().cpu().numpy(), xl)
+    assert logits3.grad.data_ptr() != logits3.data_ptr()
+    # the extension function itself: (scores, grad) with grad aliasing logits; None without grad
+    ext = ot._optimized_transducer
+    l4 = _dev(x, device).requires_grad_(True)
+    scores, grad = ext.compute_transducer_loss(logits=l4, targets=tg, logit_lengths=T,
+                                               target_lengths=U, blank=0, from_log_softmax=False,
+                                               one_sym_per_frame=False)
+    assert grad.data_ptr() == l4.data_ptr() and scores.shape == (w.N,)
+    assert np.allclose(-scores.sum().item(), loss.item(), rtol=1e-6)  # scores are +log-likelihoods
+    scores5, grad5 = ext.compute_transducer_loss(logits=_dev(x, device), targets=tg, logit_lengths=T,
+                                                 target_lengths=U, blank=0, from_log_softmax=False,
+                                                 one_sym_per_frame=False)
+    assert grad5 is None and torch.equal(scores5, scores)
+
+
+def test_gradient_flows_into_the_network_that_made_the_logits(device):
+    # logits as a non-leaf (the normal case: output of the joiner's Linear)
+    import optimized_transducer_amd as ot
+    w = workloads.tiny()
+    x = w.logits_numpy()
+    tg, T, U = _dev(w.targets, device), _dev(w.logit_lengths, device), _dev(w.target_lengths, device)
+    torch.manual_seed(0)
+    h = torch.randn(x.shape[0], 16, device=device)
+    lin = torch.nn.Linear(16, w.V).to(device)
+    loss = ot.TransducerLoss(blank=0, reduction="mean")(lin(h), tg, T, U, False)
+    loss.backward()
+    logits = lin(h).detach().cpu().numpy()
+    _, g = oracle.transducer_loss(logits.copy(), w.targets, w.logit_lengths, w.target_lengths, 0,
+                                  False, False, "mean", dtype=np.float64)
+    want_w = g.T @ h.double().cpu().numpy()
+    assert np.allclose(lin.weight.grad.cpu().numpy(), want_w, rtol=1e-3, atol=1e-4)
+    assert np.allclose(lin.bias.grad.cpu().numpy(), g.sum(0), rtol=1e-3, atol=1e-4)
+
+
+def test_argument_checks_on_the_device(device):
+    import optimized_transducer_amd as ot
+    w = workloads.tiny()
+    x = w.logits_numpy()
+    tg, T, U = _dev(w.targets, device), _dev(w.logit_lengths, device), _dev(w.target_lengths, device)
+
+    def call(**kw):
+        args = dict(logits=_dev(x, device).requires_grad_(True), targets=tg, logit_lengths=T,
+                    target_lengths=U, blank=0, from_log_softmax=False)
+        args.update(kw)
+        return args, ot.transducer_loss(**args)
+
+    bad_rows = _dev(x[:-1], device).requires_grad_(True)
+    with pytest.raises(RuntimeError, match="Expected tensor to have size %d at dimension 0" % x.shape[0]):
+        call(logits=bad_rows)
+    assert np.array_equal(bad_rows.detach().cpu().numpy(), x[:-1])  # refused before any write
+    big = w.targets.copy()
+    big[0, 0] = w.V
+    with pytest.raises(RuntimeError, match="targets.max\\(\\) vs logits.size\\(1\\) is 32 vs 32"):
+        call(targets=_dev(big, device))
+    with pytest.raises(RuntimeError, match="Expect 0 <= blank < logits.size\\(1\\)"):
+        call(blank=w.V)
+    wide = np.concatenate([w.targets, w.targets[:, :1]], 1)
+    with pytest.raises(RuntimeError, match="targets.size\\(1\\) should be equal to target_lengths.max"):
+        call(targets=_dev(wide, device))
+    with pytest.raises(RuntimeError):  # tensors on different devices
+        call(target_lengths=torch.from_numpy(w.target_lengths))
+    neg = w.targets.copy()
+    neg[1, 1] = -3
+    with pytest.raises(RuntimeError, match="targets.min"):
+        call(targets=_dev(neg, device))
+    with pytest.raises(AssertionError):
+        call(reduction="none")
+    call()  # and the good call still works afterwards
+
+
+def test_reference_test_shapes_modified_logits_vs_logsoftmax(device):
+    # test_max_symbol_per_frame.py:14-65: T=107/209, U+1=51/62, V=200, rand logits,
+    # targets in [1, V-1); log-softmax path == logits path, loss atol 1e-6 (relative to a
+    # mean loss of a few hundred: we use rel 1e-6), grads atol 1e-4
+    import optimized_transducer_amd as ot
+    rng = np.random.default_rng(20220117)
+    T = np.array([107, 209], np.int32)
+    U = np.array([50, 61], np.int32)
+    V = 200
+    tg = rng.integers(1, V - 1, size=(2, 61)).astype(np.int32)
+    x = rng.random((int((T * (U + 1)).sum()), V), dtype=np.float32)
+    a = _dev(x, device).requires_grad_(True)
+    b = _dev(x, device).requires_grad_(True)
+    dtg, dT, dU = _dev(tg, device), _dev(T, device), _dev(U, device)
+    la = ot.transducer_loss(b.log_softmax(-1), dtg, dT, dU, 0, True, one_sym_per_frame=True)
+    lb = ot.transducer_loss(a, dtg, dT, dU, 0, False, one_sym_per_frame=True)
+    la.backward()
+    lb.backward()
+    assert abs(la.item() - lb.item()) <= 1e-6 * abs(lb.item()) + 1e-6
+    assert torch.allclose(a.grad, b.grad, atol=1e-4)
+    # and both equal the oracle
+    want_loss, want = oracle.transducer_loss(x.copy(), tg, T, U, 0, False, True, "mean")
+    assert np.allclose(lb.item(), want_loss, rtol=RTOL, atol=ATOL)
+    assert np.allclose(a.grad.cpu().numpy(), want, atol=1e-4)
+
+
+# ------------------------------------------------------------------ full sizes
+FULL = [
+    ("asr", lambda: workloads.asr_batch()),
+    ("asr_logsoftmax_modified", lambda: workloads.asr_batch_logsoftmax_modified()),
+    ("largevocab", lambda: workloads.large_vocab()),
+    ("ragged", lambda: workloads.ragged()),
+    ("ragged_modified", lambda: workloads.ragged(one_sym_per_frame=True)),
+]
+
+
+@pytest.mark.parametrize("name,make", FULL, ids=[f[0] for f in FULL])
+def test_full_size_workloads(name, make, device):
+    w = make()
+    fls, osf = w.from_log_softmax, w.one_sym_per_frame
+    T, U, tg = w.logit_lengths, w.target_lengths, w.targets
+    x = w.logits_torch(device)
+    dT, dU, dtg = _dev(T, device), _dev(U, device), _dev(tg, device)
+    max_u1 = int(U.max()) + 1
+    splits, total = oracle.row_splits(T, U)
+    assert total == x.shape[0]
+
+    # oracle on a slice: utterances are independent, so the rows of any subset of
+    # utterances must equal the oracle run on that subset alone.  Take the longest
+    # lattice, the first and the last utterance, and every degenerate one.
+    sizes = T.astype(np.int64) * (U + 1)
+    pick = sorted(set([int(np.argmax(T + U)), 0, len(T) - 1]
+                      + [int(i) for i in np.where((T == 1) | (U == 0))[0][:4]]))
+    xs = torch.cat([x[splits[b]:splits[b + 1]] for b in pick]).cpu().numpy()
+    tgs = np.ascontiguousarray(tg[pick][:, :max(int(U[pick].max()), 0)])
+    s32, g32 = oracle.compute_transducer_loss(xs.copy(), tgs, T[pick], U[pick], w.blank, fls, osf)
+    s64, g64 = oracle.compute_transducer_loss(xs.copy(), tgs, T[pick], U[pick], w.blank, fls, osf,
+                                              dtype=np.float64)
+
+    work = x.clone()
+    scores, grad, st = cabi.transducer_loss(work, dtg, dT, dU, w.blank, fls, osf, max_u1,
+                                            grad=("new" if fls else "inplace"))
+    assert st.sum_tu == total and st.targets_max == tg.max() and st.target_len_max == U.max()
+    scores_np = scores.cpu().numpy()
+    assert np.isfinite(scores_np).all()
+
+    got_s = scores_np[pick]
+    got_g = torch.cat([grad[splits[b]:splits[b + 1]] for b in pick]).cpu().numpy()
+    assert np.allclose(got_s, s32, rtol=RTOL, atol=ATOL), np.abs(got_s - s32).max()
+    tol = helpers.lattice_noise_tolerance(g32, helpers.per_row(s32, T[pick], U[pick]))
+    assert (np.abs(got_g - g32) <= tol).all(), np.abs(got_g - g32).max()
+    # float64 arbiter: no further from the exact gradient than the fp32 reference arithmetic
+    assert np.abs(got_g - g64).max() <= 2 * np.abs(g32 - g64).max() + 1e-6
+
+    # size-independent properties over the whole batch
+    if fls:
+        occ = -grad.sum(1)  # node occupancies
+        assert (occ >= -1e-6).all()
+        assert (occ <= 1 + 64 * helpers.EPS32 * np.abs(scores_np).max()).all()
+        # occupancies of one frame (modified) / all frames (standard) add up per utterance
+        per_utt = np.add.reduceat(occ.double().cpu().numpy(), splits[:-1])
+        want = T.astype(np.float64) if osf else (T + U).astype(np.float64)
+        assert np.allclose(per_utt, want, rtol=5e-3)
+        assert torch.equal(work, x)  # log-softmax input is never written
+    else:
+        rs = grad.sum(1).abs().max().item()
+        assert rs < 1e-3, rs  # rows of d loss / d logits sum to zero
+        assert grad.data_ptr() == work.data_ptr()
+    # entries are probabilities up to the fp32 noise of exp(arguments of size |loss|)
+    assert grad.abs().max().item() <= 1 + 64 * helpers.EPS32 * np.abs(scores_np).max()
+
+    # same bits on a second run (no atomics, no data races)
+    work2 = x.clone()
+    scores2, grad2, _ = cabi.transducer_loss(work2, dtg, dT, dU, w.blank, fls, osf, max_u1,
+                                             grad=("new" if fls else "inplace"))
+    assert torch.equal(scores2, scores) and torch.equal(grad2, grad)

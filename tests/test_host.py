@@ -1,0 +1,164 @@
+"""Host-side logic that needs no GPU: the C ABI surface, the drop-in Python
+surface, and the argument checks (which mirror
+optimized_transducer/csrc/transducer-loss.cc:33-66 and are compared message by
+message with the compiled reference where oracle/_ref has been built)."""
+import ctypes
+import inspect
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import cabi
+from oracle import ref_loader
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ----------------------------------------------------------------- C ABI
+def declared_symbols():
+    text = open(cabi.HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ot_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_symbol_the_header_declares():
+    names = declared_symbols()
+    assert {"ot_row_splits", "ot_log_probs", "ot_alpha_beta", "ot_gradient",
+            "ot_transducer_loss"} <= set(names)
+    lib = ctypes.CDLL(cabi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_c_abi_rejects_bad_arguments_before_touching_the_device():
+    L = cabi.lib()
+    null = ctypes.c_void_p(0)
+    i32, i64 = ctypes.c_int32, ctypes.c_int64
+    assert L.ot_row_splits(null, null, null, i32(4), i32(3), null, null, null) == -1
+    assert L.ot_row_ids(null, i32(1), i64(5), null, null) == -1
+    assert L.ot_log_probs(null, null, null, null, i32(1), i32(0), i64(4), i32(8), i32(0), i32(0),
+                          null, null, null) == -1
+    one = ctypes.c_void_p(16)  # never dereferenced: the size checks fail first
+    assert L.ot_alpha_beta(one, one, one, one, i32(1), i32(2000), i32(0), one, one, one, one,
+                           null) == -2  # OT_E_TOO_LONG
+    assert L.ot_log_probs(one, one, one, one, i32(1), i32(1), i64(4), i32(8), i32(9), i32(0), one,
+                          one, null) == -1  # blank >= V
+    assert L.ot_gradient(null, null, null, null, null, null, null, null, null, i32(1), i32(0),
+                         i64(1), i32(4), i32(0), i32(0), i32(0), ctypes.c_float(1), null, null,
+                         null) == -1
+    assert L.ot_workspace_bytes(i32(0), i64(10)) == 0
+    n1 = L.ot_workspace_bytes(i32(4), i64(1000))
+    n2 = L.ot_workspace_bytes(i32(4), i64(2000))
+    assert 1000 * 44 <= n1 < n2 < 2000 * 44 + 4096 * 8
+    assert L.ot_gradient_scratch_bytes(i64(10)) == 240
+    assert b"OT_MAX_U1" in L.ot_error_string(-2)
+    assert L.ot_error_string(0) == b"success"
+
+
+# ------------------------------------------------------------ Python surface
+def test_python_entry_points_keep_the_reference_signatures():
+    import optimized_transducer_amd as ot
+    # optimized_transducer/python/optimized_transducer/transducer_loss.py:312-321
+    sig = inspect.signature(ot.transducer_loss)
+    assert list(sig.parameters) == ["logits", "targets", "logit_lengths", "target_lengths", "blank",
+                                    "from_log_softmax", "one_sym_per_frame", "reduction"]
+    assert sig.parameters["one_sym_per_frame"].default is False
+    assert sig.parameters["reduction"].default == "mean"
+    assert sig.parameters["from_log_softmax"].default is inspect.Parameter.empty
+    # transducer_loss.py:174, :190-198
+    init = inspect.signature(ot.TransducerLoss.__init__)
+    assert list(init.parameters) == ["self", "blank", "reduction"]
+    assert init.parameters["reduction"].default == "mean"
+    fwd = inspect.signature(ot.TransducerLoss.forward)
+    assert list(fwd.parameters) == ["self", "logits", "targets", "logit_lengths", "target_lengths",
+                                    "from_log_softmax", "one_sym_per_frame"]
+    assert fwd.parameters["one_sym_per_frame"].default is False
+    m = ot.TransducerLoss(blank=0, reduction="sum")  # the reference's class cannot be called
+    assert isinstance(m, torch.nn.Module) and m.blank == 0 and m.reduction == "sum"
+    # optimized_transducer.cc:14-18: seven keyword-nameable arguments, no defaults
+    doc = ot._optimized_transducer.compute_transducer_loss.__doc__
+    for kw in ("logits", "targets", "logit_lengths", "target_lengths", "blank", "from_log_softmax",
+               "one_sym_per_frame"):
+        assert kw + ":" in doc
+
+
+def _good():
+    T = torch.tensor([3, 4], dtype=torch.int32)
+    U = torch.tensor([2, 1], dtype=torch.int32)
+    targets = torch.tensor([[1, 2], [2, 1]], dtype=torch.int32)
+    logits = torch.randn(3 * 3 + 4 * 2, 5)
+    return dict(logits=logits, targets=targets, logit_lengths=T, target_lengths=U, blank=0,
+                from_log_softmax=False, one_sym_per_frame=False)
+
+
+def _mutations():
+    def m(**kw):
+        a = _good()
+        a.update(kw)
+        return a
+    g = _good()
+    return {
+        "logits dtype": m(logits=g["logits"].double()),
+        "targets dtype": m(targets=g["targets"].long()),
+        "logit_lengths dtype": m(logit_lengths=g["logit_lengths"].long()),
+        "target_lengths dtype": m(target_lengths=g["target_lengths"].short()),
+        "non contiguous": m(logits=torch.randn(5, 17).t()),
+        "logits dim": m(logits=torch.randn(17 * 5)),
+        "targets dim": m(targets=torch.tensor([1, 2], dtype=torch.int32)),
+        "lengths size": m(logit_lengths=torch.tensor([3, 4, 5], dtype=torch.int32)),
+        "sum_TU": m(logits=torch.randn(16, 5)),
+        "targets max": m(targets=torch.tensor([[1, 5], [2, 1]], dtype=torch.int32)),
+        "blank high": m(blank=5),
+        "blank negative": m(blank=-1),
+        "targets cols": m(targets=torch.tensor([[1, 2, 3], [2, 1, 1]], dtype=torch.int32)),
+    }
+
+
+def _message(fn, args):
+    with pytest.raises(RuntimeError) as e:
+        fn(**args)
+    return str(e.value).split("\n")[0]
+
+
+@pytest.mark.parametrize("name", sorted(_mutations()))
+def test_argument_checks_raise_like_the_reference(name):
+    import optimized_transducer_amd as ot
+    args = _mutations()[name]
+    msg = _message(ot._optimized_transducer.compute_transducer_loss, args)
+    assert "no CPU implementation" not in msg, "bad argument went undetected: " + msg
+    ref = ref_loader.load()
+    if ref is not None:
+        want = _message(ref.compute_transducer_loss, _mutations()[name])
+        assert msg == want
+
+
+def test_valid_cpu_tensors_are_refused_not_computed():
+    import optimized_transducer_amd as ot
+    msg = _message(ot._optimized_transducer.compute_transducer_loss, _good())
+    assert "no CPU implementation" in msg
+    with pytest.raises(RuntimeError):
+        ot.transducer_loss(**{k: v for k, v in _good().items()}, reduction="sum")
+
+
+def test_reduction_none_is_rejected_like_the_reference():
+    import optimized_transducer_amd as ot
+    with pytest.raises(AssertionError):  # transducer_loss.py:133
+        ot.transducer_loss(**_good(), reduction="none")
+
+
+def test_product_never_imports_the_oracle():
+    for root, _, files in os.walk(os.path.join(ROOT, "optimized_transducer_amd")):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(root, f)).read()
+                assert "oracle" not in text.lower(), os.path.join(root, f)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert p.returncode != 0 and "one GPU" in (p.stderr + p.stdout)
