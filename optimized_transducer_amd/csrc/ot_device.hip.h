@@ -213,6 +213,12 @@ __device__ __forceinline__ Cell decode_row(const BlockUtterances &bu, int64_t ro
 }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+// cache-policy operand of the raw buffer builtins: bit 1 = non-temporal
+#ifndef OT_AUX_STREAM
+#define OT_AUX_STREAM 2
+#endif
+constexpr int kAuxStream = OT_AUX_STREAM;
 
 // VEC floats of a row.  The (rows, V) arrays are streamed once per kernel and
 // never re-read by the same kernel, so their loads and stores carry the
@@ -232,6 +238,20 @@ template <> struct Vec<4> {
     const f32x4 x = {v[0], v[1], v[2], v[3]};
     *reinterpret_cast<f32x4 *>(p) = x;
   }
+  __device__ __forceinline__ void load_lds(const float *p) {
+    const f32x4 x = *reinterpret_cast<const f32x4 *>(p);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  }
+  // streaming (non-temporal) buffer access: out-of-range reads give 0, writes vanish
+  __device__ __forceinline__ void load_buffer(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
+    const f32x4 x = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, kAuxStream));
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  }
+  __device__ __forceinline__ void store_buffer(__amdgpu_buffer_rsrc_t r, unsigned byte_off) const {
+    const f32x4 x = {v[0], v[1], v[2], v[3]};
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, x), r, byte_off, 0, kAuxStream);
+  }
+  __device__ __forceinline__ void store_lds(float *p) const { store(p); }
   // for flat, line-aligned streams only: a non-temporal store of a partial
   // cache line is much slower than a cached one
   __device__ __forceinline__ void store_stream(float *p) const {
@@ -248,6 +268,14 @@ template <> struct Vec<1> {
   __device__ __forceinline__ void load(const float *p) { v[0] = __builtin_nontemporal_load(p); }
   __device__ __forceinline__ void store(float *p) const { *p = v[0]; }
   __device__ __forceinline__ void store_stream(float *p) const { __builtin_nontemporal_store(v[0], p); }
+  __device__ __forceinline__ void load_lds(const float *p) { v[0] = *p; }
+  __device__ __forceinline__ void load_buffer(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
+    v[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, kAuxStream));
+  }
+  __device__ __forceinline__ void store_buffer(__amdgpu_buffer_rsrc_t r, unsigned byte_off) const {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v[0]), r, byte_off, 0, kAuxStream);
+  }
+  __device__ __forceinline__ void store_lds(float *p) const { *p = v[0]; }
 };
 
 }  // namespace ot

@@ -111,17 +111,31 @@ __global__ void row_ids_kernel(const int32_t *__restrict__ row_splits, int N, in
 // ---------------------------------------------------------------------------
 // per-row log-sum-exp + blank/target gather, one pass over the logits
 // ---------------------------------------------------------------------------
-// Row r of a workgroup's span is handled by lanes [g*L, g*L+L) of one wave
-// (g = r mod 64/L).  Vector j of the row (VEC floats) lives in lane j mod L,
-// register slot (j / L) mod K, chunk j / (L*K).
+// A group of L lanes reduces one row, so a wave reduces G = 64/L rows per pass;
+// vector j of a row (VEC floats) is held by lane j mod L of the group in
+// register slot j / L.
+//
+// Memory side: the G rows of a pass are contiguous, so the wave reads them as
+// one flat span (lane i takes vectors i, i+64, ...: each load instruction covers
+// an aligned, contiguous 1 KiB, which a 2000-byte row cut into 256-byte pieces
+// does not) and re-shapes the span into the row-group layout through a
+// wave-private LDS buffer.  The loads of the next pass are issued before the
+// current pass is reduced.  The blank/target gather then reads LDS, not HBM.
+// Rows longer than L*K vectors (L = 64, so flat and row-group layout coincide)
+// stream through registers in chunks with a running (max, scaled sum).
+#ifndef OT_LSE_WAVES_PER_SIMD
+#define OT_LSE_WAVES_PER_SIMD 1
+#endif
 template <int VEC, int L, int K>
-__global__ __launch_bounds__(kBlock) void lse_gather_kernel(
+__global__ __launch_bounds__(kBlock, OT_LSE_WAVES_PER_SIMD) void lse_gather_kernel(
     const float *__restrict__ logits, const int32_t *__restrict__ targets,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
     int N, int targets_cols, int64_t rows, int V, int blank, int rows_per_block,
     float *__restrict__ den, float *__restrict__ lp) {
   constexpr int G = kWave / L;
+  constexpr bool kStaged = G > 1;
   __shared__ BlockUtterances bu;
+  __shared__ __attribute__((aligned(16))) float s_stage[kStaged ? kWavesPerBlock * kWave * K * VEC : 4];
   const int64_t row_first = (int64_t)blockIdx.x * rows_per_block;
   const int64_t row_end = min(rows, row_first + rows_per_block);
   bu.load(row_splits, N, row_first, row_end - 1);
@@ -130,21 +144,49 @@ __global__ __launch_bounds__(kBlock) void lse_gather_kernel(
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sub = lane % L, g = lane / L;
   const int nvec = V / VEC;  // VEC divides V by construction of the launch
+  const bool whole_row = nvec <= L * K;
+  float *stage = s_stage + (kStaged ? wave * (kWave * K * VEC) : 0);
 
-  for (int64_t base = row_first + (int64_t)wave * G; base < row_end; base += kWavesPerBlock * G) {
+  // flat span of the pass that starts at row `base`: registers a[].  The
+  // workgroup's rows are one raw buffer, so the tail of the last span (rows past
+  // row_end) reads as zeros without a bounds branch.
+  const __amdgpu_buffer_rsrc_t block_buf =
+      make_buffer(logits + row_first * (int64_t)V, (unsigned)((row_end - row_first) * V * 4));
+  Vec<VEC> a[K];
+  auto issue_span = [&](int64_t base) {
+    const unsigned off0 = (unsigned)(base - row_first) * (unsigned)V * 4u;
+#pragma unroll
+    for (int k = 0; k < K; ++k) a[k].load_buffer(block_buf, off0 + (unsigned)(k * kWave + lane) * (VEC * 4u));
+  };
+
+  int64_t base = row_first + (int64_t)wave * G;
+  if (kStaged && whole_row && base < row_end) issue_span(base);
+
+  for (; base < row_end; base += kWavesPerBlock * G) {
     const int64_t row = base + g;
     const bool active = row < row_end;
     const float *p = logits + (active ? row : row_first) * (int64_t)V;
 
     float m, s;
-    if (nvec <= L * K) {
+    if (whole_row) {
       // whole row in registers: exact max first, then one exp per element
       Vec<VEC> x[K];
+      if (kStaged) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) a[k].store_lds(stage + (k * kWave + lane) * VEC);
+        issue_span(base + kWavesPerBlock * G);  // past row_end: all zeros, never used
+      }
       float cm = OT_NEG_INF;
 #pragma unroll
       for (int k = 0; k < K; ++k) {
         const int j = k * L + sub;
-        if (j < nvec) {
+        if (kStaged) {
+          // always inside the wave's buffer; slots past the row are masked
+          x[k].load_lds(stage + (g * nvec + j) * VEC);
+          const bool keep = (j < nvec) & active;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) x[k].v[e] = keep ? x[k].v[e] : OT_NEG_INF;
+        } else if (j < nvec) {
           x[k].load(p + (int64_t)j * VEC);
         } else {
 #pragma unroll
@@ -212,7 +254,9 @@ __global__ __launch_bounds__(kBlock) void lse_gather_kernel(
             ok = (unsigned)col < (unsigned)V;
           }
         }
-        lp[2 * row + sub] = ok ? p[col] - d : OT_NEG_INF;
+        float x = 0.f;
+        if (ok) x = (kStaged && whole_row) ? stage[g * V + col] : p[col];
+        lp[2 * row + sub] = ok ? x - d : OT_NEG_INF;
       }
     }
   }
@@ -468,13 +512,18 @@ __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
   const int64_t base = (int64_t)blockIdx.x * (kGradUnroll * kBlock);
   const int64_t row_base = base / nvec;
   const int rem_base = (int)(base - row_base * nvec);
+  // the workgroup's units as raw buffers: the tail of the last workgroup needs no branch
+  const unsigned span_bytes =
+      (unsigned)min((int64_t)(kGradUnroll * kBlock), nunits - base) * (VEC * 4u);
+  const __amdgpu_buffer_rsrc_t in_buf = make_buffer(FLS ? grad : logits + base * VEC, span_bytes);
+  const __amdgpu_buffer_rsrc_t out_buf = make_buffer(grad + base * VEC, span_bytes);
 
   Vec<VEC> x[kGradUnroll];
   int rows[kGradUnroll], col0[kGradUnroll];
 #pragma unroll
   for (int k = 0; k < kGradUnroll; ++k) {
     const int local = k * kBlock + (int)threadIdx.x;
-    if (!FLS && base + local < nunits) x[k].load(logits + (base + local) * VEC);
+    if (!FLS) x[k].load_buffer(in_buf, (unsigned)local * (VEC * 4u));
     // idx < nvec + 1024 is exact in float; one correction step fixes the quotient
     const int idx = rem_base + local;
     int q = (int)((float)idx * inv_nvec);
@@ -482,11 +531,11 @@ __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
     rows[k] = q;
     col0[k] = (idx - q * nvec) * VEC;
   }
+  const int64_t last_row = (nunits - 1) / nvec;
 #pragma unroll
   for (int k = 0; k < kGradUnroll; ++k) {
     const int local = k * kBlock + (int)threadIdx.x;
-    if (base + local >= nunits) continue;
-    const int64_t row = row_base + rows[k];
+    const int64_t row = min(row_base + rows[k], last_row);
     const float4 f = coef_f[row];
     const int2 ci = coef_i[row];
     Vec<VEC> y;
@@ -518,7 +567,7 @@ __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
         for (int e = 0; e < VEC; ++e) y.v[e] *= scale;
       }
     }
-    y.store_stream(grad + (base + local) * VEC);
+    y.store_buffer(out_buf, (unsigned)local * (VEC * 4u));
   }
 }
 
@@ -552,6 +601,9 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const float4 *__restrict__
 // ---------------------------------------------------------------------------
 // host side: geometry and dispatch
 // ---------------------------------------------------------------------------
+#ifndef OT_TUNE_BLOCK_BYTES
+#define OT_TUNE_BLOCK_BYTES (256 * 1024)
+#endif
 struct RowTiling {
   int vec, L, K, rows_per_block;
 };
@@ -569,7 +621,7 @@ static RowTiling pick_tiling(int V, bool aligned16) {
   t.K = K;
   // about 256 KiB of logits per workgroup, a whole number of wave passes
   const int pass = kWavesPerBlock * (kWave / L);
-  int64_t want = (256 * 1024) / ((int64_t)V * 4);
+  int64_t want = (OT_TUNE_BLOCK_BYTES) / ((int64_t)V * 4);
   int rpb = (int)((want / pass) * pass);
   if (rpb < pass) rpb = pass;
   if (rpb > kMaxRowsPerBlock) rpb = kMaxRowsPerBlock;
