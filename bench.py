@@ -22,6 +22,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs scaled by the library's 1 GiB copy kernel (x2.000 / x1.000);
+# summary and commands in profiles/hbm_traffic_bench_asr_N32_V500.md.  Valid for
+# this workload and the kernel's current access pattern only.
+MEASURED_TRAFFIC_BYTES = {("asr_N32_V500", "grad_logits"): 3.0495e9}
+
 
 def make_workload(name):
     import workloads
@@ -106,6 +112,10 @@ def main():
     ap.add_argument("--workload", default="asr")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch the library's plain copy kernel on 1 GiB (read 1 GiB + "
+                         "write 1 GiB) three times, as a known-size reference for profiler "
+                         "byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build measures one GPU only (got --gpus %d); "
@@ -132,6 +142,19 @@ def main():
                                   w.one_sym_per_frame, w.reduction)
         loss.backward()
         return loss
+
+    if args.calibrate_copy:
+        import ctypes
+        lib = ctypes.CDLL(os.path.join(ROOT, "optimized_transducer_amd", "libot_transducer.so"))
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            rc = lib.ot_copy_floats(ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()),
+                                    ctypes.c_int64(src.numel()),
+                                    ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+            assert rc == 0, rc
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(W):
         step(pristine.clone())
@@ -180,9 +203,12 @@ def main():
                 kernels[name]["achieved_GBps"] = alg[name] / (avg * 1e-3) / 1e9
         dom = "grad_logsoftmax" if w.from_log_softmax else "grad_logits"
         achieved = kernels[dom]["achieved_GBps"]
-        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": achieved,
+        kernel_name = "grad_flat_kernel<%d,%s>" % (4 if w.V % 4 == 0 else 1,
+                                                    "true" if w.from_log_softmax else "false")
+        out["roofline"] = {"bound": "hbm", "kernel": kernel_name, "achieved": achieved,
                            "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                           "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                           "frac": achieved / HBM_PEAK_GBPS,
+                           "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, dom)),
                            "avg_launch_ms": kernels[dom]["avg_ms"],
                            "algorithmic_bytes_per_launch": alg[dom]}
         out["kernels"] = kernels

@@ -99,8 +99,8 @@ int ot_alpha_beta(const float *lp, const int32_t *logit_lengths,
  * grad_scale.
  * from_log_softmax == 0: ComputeGradient / ComputeGradientOneSymPerFrame
  *   (cuda.cu:308-346, kernels.cu:522-651); `grad` may be the same pointer as
- *   `logits` (the reference's in-place mode, cuda.cu:449) - each row is read
- *   completely before it is written.  lp is not used (may be NULL).
+ *   `logits` (the reference's in-place mode, cuda.cu:449) - every element is
+ *   read before it is written, by the same thread.  lp is not used (may be NULL).
  * from_log_softmax != 0: ComputeGradientForLogSoftmax(+OneSymPerFrame)
  *   (cuda.cu:364-400, kernels.cu:653-779); `grad` must not alias `logits`;
  *   only lp is read, logits and den may be NULL.
@@ -116,6 +116,22 @@ int ot_gradient(const float *logits, const float *lp, const float *den,
                 int64_t rows, int32_t V, int32_t blank,
                 int32_t from_log_softmax, int32_t one_sym_per_frame,
                 float grad_scale, void *row_scratch, float *grad, void *stream);
+
+/* The two launches of ot_gradient on their own, for callers that want to time
+ * or schedule them separately: per-row coefficients into `row_scratch`
+ * (same arguments and meaning as in ot_gradient), then the flat pass that
+ * reads `logits` and writes `grad`. */
+int ot_row_coefficients(const float *lp, const float *den, const float *alpha,
+                        const float *beta, const int32_t *targets,
+                        const int32_t *logit_lengths,
+                        const int32_t *target_lengths, const int32_t *row_splits,
+                        int32_t N, int32_t targets_cols, int64_t rows,
+                        int32_t blank, int32_t from_log_softmax,
+                        int32_t one_sym_per_frame, float grad_scale,
+                        void *row_scratch, void *stream);
+int ot_gradient_apply(const float *logits, const void *row_scratch, int64_t rows,
+                      int32_t V, int32_t from_log_softmax, float grad_scale,
+                      float *grad, void *stream);
 
 /* Bytes of 16-byte aligned device scratch ot_gradient needs in `row_scratch`
  * (per-row coefficients, 24 bytes per packed row). */

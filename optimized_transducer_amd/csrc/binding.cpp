@@ -230,6 +230,10 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   const int32_t max_u1 = st.target_len_max + 1;
   TORCH_CHECK(max_u1 <= OT_MAX_U1, "target_lengths.max() + 1 is ", max_u1,
               ", which exceeds the supported ", OT_MAX_U1);
+  // the lattice kernel addresses one utterance's cells with 32-bit byte offsets
+  TORCH_CHECK(((int64_t)st.logit_len_max + 1300) * max_u1 < ((int64_t)1 << 29),
+              "an utterance with T = ", st.logit_len_max, " and up to ", max_u1,
+              " lattice columns is too large for the lattice kernel");
 
   torch::Tensor scores = torch::empty({N}, logits.options());
   {
@@ -243,11 +247,17 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
     // cpu.cc:803 / cuda.cu:444: new tensor for log-softmax input;
     // cpu.cc:814 / cuda.cu:449: the logits buffer itself otherwise.
     gradient = from_log_softmax ? torch::empty_like(logits) : logits;
-    ScopedTimer timer(from_log_softmax ? "grad_logsoftmax" : "grad_logits", stream);
-    OT_CHECK(ot_gradient(p_logits, lp, den, alpha, beta, p_targets, p_T, p_U, row_splits,
-                         (int32_t)N, (int32_t)S, rows, (int32_t)V, blank, from_log_softmax,
-                         one_sym_per_frame, (float)grad_scale, w + off_coef,
-                         gradient.data_ptr<float>(), stream));
+    {
+      ScopedTimer timer("row_coeff", stream);
+      OT_CHECK(ot_row_coefficients(lp, den, alpha, beta, p_targets, p_T, p_U, row_splits,
+                                   (int32_t)N, (int32_t)S, rows, blank, from_log_softmax,
+                                   one_sym_per_frame, (float)grad_scale, w + off_coef, stream));
+    }
+    {
+      ScopedTimer timer(from_log_softmax ? "grad_logsoftmax" : "grad_logits", stream);
+      OT_CHECK(ot_gradient_apply(p_logits, w + off_coef, rows, (int32_t)V, from_log_softmax,
+                                 (float)grad_scale, gradient.data_ptr<float>(), stream));
+    }
   }
   if (gradient.defined()) return {scores, gradient};
   return {scores, torch::nullopt};

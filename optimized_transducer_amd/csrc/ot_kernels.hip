@@ -726,36 +726,42 @@ int ot_alpha_beta(const float *lp, const int32_t *logit_lengths, const int32_t *
   return launch_status();
 }
 
-int ot_gradient(const float *logits, const float *lp, const float *den, const float *alpha,
-                const float *beta, const int32_t *targets, const int32_t *logit_lengths,
-                const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
-                int32_t targets_cols, int64_t rows, int32_t V, int32_t blank,
-                int32_t from_log_softmax, int32_t one_sym_per_frame, float grad_scale,
-                void *row_scratch, float *grad, void *stream) {
-  if (!alpha || !beta || !logit_lengths || !target_lengths || !row_splits || !grad ||
-      !row_scratch || N <= 0 || rows <= 0 || rows > INT32_MAX || V <= 0 || blank < 0 ||
-      blank >= V || targets_cols < 0 || (targets_cols > 0 && !targets))
+int ot_row_coefficients(const float *lp, const float *den, const float *alpha, const float *beta,
+                        const int32_t *targets, const int32_t *logit_lengths,
+                        const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
+                        int32_t targets_cols, int64_t rows, int32_t blank,
+                        int32_t from_log_softmax, int32_t one_sym_per_frame, float grad_scale,
+                        void *row_scratch, void *stream) {
+  if (!alpha || !beta || !logit_lengths || !target_lengths || !row_splits || !row_scratch ||
+      N <= 0 || rows <= 0 || rows > INT32_MAX || blank < 0 || targets_cols < 0 ||
+      (targets_cols > 0 && !targets) || (from_log_softmax ? !lp : !den))
     return OT_E_BAD_ARG;
-  if (from_log_softmax ? (!lp || grad == logits) : (!logits || !den)) return OT_E_BAD_ARG;
+  if (reinterpret_cast<uintptr_t>(row_scratch) & 15) return OT_E_MISALIGNED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float4 *coef_f = static_cast<float4 *>(row_scratch);
+  int2 *coef_i = reinterpret_cast<int2 *>(coef_f + rows);
+  const dim3 grid((unsigned)((rows + kBlock - 1) / kBlock));
+  if (from_log_softmax)
+    hipLaunchKernelGGL(row_coeff_kernel<true>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
+                       targets, logit_lengths, target_lengths, row_splits, N, targets_cols, rows,
+                       blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
+  else
+    hipLaunchKernelGGL(row_coeff_kernel<false>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
+                       targets, logit_lengths, target_lengths, row_splits, N, targets_cols, rows,
+                       blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
+  return launch_status();
+}
+
+int ot_gradient_apply(const float *logits, const void *row_scratch, int64_t rows, int32_t V,
+                      int32_t from_log_softmax, float grad_scale, float *grad, void *stream) {
+  if (!row_scratch || !grad || rows <= 0 || rows > INT32_MAX || V <= 0) return OT_E_BAD_ARG;
+  if (from_log_softmax ? grad == logits : !logits) return OT_E_BAD_ARG;
   if ((reinterpret_cast<uintptr_t>(grad) & 3) || (reinterpret_cast<uintptr_t>(logits) & 3) ||
       (reinterpret_cast<uintptr_t>(row_scratch) & 15))
     return OT_E_MISALIGNED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  float4 *coef_f = static_cast<float4 *>(row_scratch);
-  int2 *coef_i = reinterpret_cast<int2 *>(coef_f + rows);
-  {
-    const dim3 grid((unsigned)((rows + kBlock - 1) / kBlock));
-    if (from_log_softmax)
-      hipLaunchKernelGGL(row_coeff_kernel<true>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
-                         targets, logit_lengths, target_lengths, row_splits, N, targets_cols, rows,
-                         blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
-    else
-      hipLaunchKernelGGL(row_coeff_kernel<false>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
-                         targets, logit_lengths, target_lengths, row_splits, N, targets_cols, rows,
-                         blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
-    const int rc = launch_status();
-    if (rc) return rc;
-  }
+  const float4 *coef_f = static_cast<const float4 *>(row_scratch);
+  const int2 *coef_i = reinterpret_cast<const int2 *>(coef_f + rows);
   const bool aligned = is_aligned16(grad) && (from_log_softmax || is_aligned16(logits));
   const int vec = (aligned && V % 4 == 0) ? 4 : 1;
   const int nvec = V / vec;
@@ -775,6 +781,20 @@ int ot_gradient(const float *logits, const float *lp, const float *den, const fl
   }
 #undef OT_LAUNCH_GRAD
   return launch_status();
+}
+
+int ot_gradient(const float *logits, const float *lp, const float *den, const float *alpha,
+                const float *beta, const int32_t *targets, const int32_t *logit_lengths,
+                const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
+                int32_t targets_cols, int64_t rows, int32_t V, int32_t blank,
+                int32_t from_log_softmax, int32_t one_sym_per_frame, float grad_scale,
+                void *row_scratch, float *grad, void *stream) {
+  if (V <= 0 || blank >= V) return OT_E_BAD_ARG;
+  int rc = ot_row_coefficients(lp, den, alpha, beta, targets, logit_lengths, target_lengths,
+                               row_splits, N, targets_cols, rows, blank, from_log_softmax,
+                               one_sym_per_frame, grad_scale, row_scratch, stream);
+  if (rc) return rc;
+  return ot_gradient_apply(logits, row_scratch, rows, V, from_log_softmax, grad_scale, grad, stream);
 }
 
 size_t ot_gradient_scratch_bytes(int64_t rows) {
