@@ -55,10 +55,13 @@ typedef struct ot_batch_status {
  * cuda.cu:411-414 and the reductions at transducer-loss.cc:49,53,62.
  * row_splits: (N+1,) int32, row_splits[0] = 0, int32 wrap-around like the
  * reference; status: one ot_batch_status.  targets may be NULL when
- * targets_cols == 0. */
+ * targets_cols == 0.  row_splits_mirror (may be NULL) receives a second copy
+ * of row_splits; it and `status` may be device-visible pinned host memory, so
+ * that the host can read both after waiting for an event on `stream`. */
 int ot_row_splits(const int32_t *logit_lengths, const int32_t *target_lengths,
                   const int32_t *targets, int32_t N, int32_t targets_cols,
-                  int32_t *row_splits, ot_batch_status *status, void *stream);
+                  int32_t *row_splits, int32_t *row_splits_mirror,
+                  ot_batch_status *status, void *stream);
 
 /* Row -> utterance map, (rows,) int32.  Replaces RowSplitsToRowIds /
  * mgpu::load_balance_search (cuda.cu:40-59).  The kernels below do not need
@@ -82,6 +85,14 @@ int ot_log_probs(const float *logits, const int32_t *targets,
                  int32_t blank, int32_t from_log_softmax, float *den, float *lp,
                  void *stream);
 
+/* ot_log_probs restricted to rows [row_begin, row_end) of the same arrays
+ * (any row boundary; utterances need not be complete). */
+int ot_log_probs_range(const float *logits, const int32_t *targets,
+                       const int32_t *target_lengths, const int32_t *row_splits,
+                       int32_t N, int32_t targets_cols, int64_t rows, int32_t V,
+                       int32_t blank, int32_t from_log_softmax, int64_t row_begin,
+                       int64_t row_end, float *den, float *lp, void *stream);
+
 /* Forward and backward lattice variables, both directions in one launch.
  * Replaces ComputeAlpha / ComputeBeta and their one-symbol-per-frame twins
  * (cuda.cu:162-306, kernels.cu:200-313, kernels.cu:415-519).
@@ -94,6 +105,15 @@ int ot_alpha_beta(const float *lp, const int32_t *logit_lengths,
                   int32_t N, int32_t max_u1, int32_t one_sym_per_frame,
                   float *alpha, float *beta, float *scores_alpha,
                   float *scores_beta, void *stream);
+
+/* ot_alpha_beta restricted to utterances [utt_begin, utt_end); all arrays keep
+ * their full-batch indexing. */
+int ot_alpha_beta_range(const float *lp, const int32_t *logit_lengths,
+                        const int32_t *target_lengths, const int32_t *row_splits,
+                        int32_t N, int32_t max_u1, int32_t one_sym_per_frame,
+                        int32_t utt_begin, int32_t utt_end, float *alpha,
+                        float *beta, float *scores_alpha, float *scores_beta,
+                        void *stream);
 
 /* Gradient of the negative log-likelihood w.r.t. the rows of `logits`, times
  * grad_scale.
@@ -132,6 +152,27 @@ int ot_row_coefficients(const float *lp, const float *den, const float *alpha,
 int ot_gradient_apply(const float *logits, const void *row_scratch, int64_t rows,
                       int32_t V, int32_t from_log_softmax, float grad_scale,
                       float *grad, void *stream);
+
+/* The same two launches restricted to rows [row_begin, row_end) (whole
+ * utterances); `rows` stays the extent of the arrays.  Together with
+ * ot_log_probs_range and ot_alpha_beta_range this lets a caller run the
+ * latency-bound lattice kernel of one part of the batch on a second stream
+ * while the streaming kernels of another part use the memory system. */
+int ot_row_coefficients_range(const float *lp, const float *den,
+                              const float *alpha, const float *beta,
+                              const int32_t *targets,
+                              const int32_t *logit_lengths,
+                              const int32_t *target_lengths,
+                              const int32_t *row_splits, int32_t N,
+                              int32_t targets_cols, int64_t rows, int32_t blank,
+                              int32_t from_log_softmax,
+                              int32_t one_sym_per_frame, float grad_scale,
+                              int64_t row_begin, int64_t row_end,
+                              void *row_scratch, void *stream);
+int ot_gradient_apply_range(const float *logits, const void *row_scratch,
+                            int64_t rows, int32_t V, int32_t from_log_softmax,
+                            float grad_scale, int64_t row_begin, int64_t row_end,
+                            float *grad, void *stream);
 
 /* Bytes of 16-byte aligned device scratch ot_gradient needs in `row_scratch`
  * (per-row coefficients, 24 bytes per packed row). */

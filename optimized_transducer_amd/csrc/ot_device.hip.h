@@ -134,12 +134,25 @@ __device__ __forceinline__ float log_add(float a, float b) {
 __device__ __forceinline__ float log_add_fast(float a, float b) {
   constexpr float kLog2e = 1.44269502162933349609375f;
   constexpr float kLn2 = 0.693147182464599609375f;
-  const bool lt = a < b;
-  const float hi = lt ? b : a;
-  const float diff = lt ? (a - b) : (b - a);
+  // smaller - larger = -|a - b| (the sign and abs fold into operand modifiers);
+  // (-inf, -inf) still gives a NaN difference, which fails the threshold test
+  // below like in the reference
+  const float hi = __builtin_fmaxf(a, b);
+  const float diff = -__builtin_fabsf(a - b);
   const float e = __builtin_amdgcn_exp2f(diff * kLog2e);
   const float l = __builtin_amdgcn_logf(1.0f + e) * kLn2;
   return hi + ((diff >= kMinLogDiff) ? l : 0.0f);
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
+// for every outstanding global load and store of the wave, which would drain
+// the lattice sweep's prefetch ring at each barrier; here only the LDS counter
+// (lgkmcnt) is waited for.  simm16 0xC07F = vmcnt 63, expcnt 7, lgkmcnt 0.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // Raw buffer view of a device array: loads beyond `bytes` return 0 and stores

@@ -34,7 +34,8 @@ constexpr int kPrepThreads = 256;
 __global__ __launch_bounds__(kPrepThreads) void prepare_kernel(
     const int32_t *__restrict__ logit_lengths, const int32_t *__restrict__ target_lengths,
     const int32_t *__restrict__ targets, int N, int targets_cols,
-    int32_t *__restrict__ row_splits, ot_batch_status *__restrict__ status) {
+    int32_t *__restrict__ row_splits, int32_t *__restrict__ row_splits_mirror,
+    ot_batch_status *__restrict__ status) {
   __shared__ int s_red[6];
   __shared__ long long s_total;
   const int tid = threadIdx.x;
@@ -59,11 +60,16 @@ __global__ __launch_bounds__(kPrepThreads) void prepare_kernel(
         if (tid >= ofs) v += o;
       }
       // int32 wrap-around like cumsum(int32) of the reference
-      if (i < N) row_splits[i + 1] = (int32_t)(uint32_t)(unsigned long long)(carry + v);
+      if (i < N) {
+        const int32_t split = (int32_t)(uint32_t)(unsigned long long)(carry + v);
+        row_splits[i + 1] = split;
+        if (row_splits_mirror) row_splits_mirror[i + 1] = split;
+      }
       carry += __shfl(v, kWave - 1, kWave);
     }
     if (tid == 0) {
       row_splits[0] = 0;
+      if (row_splits_mirror) row_splits_mirror[0] = 0;
       s_total = carry;
     }
   }
@@ -130,13 +136,14 @@ template <int VEC, int L, int K>
 __global__ __launch_bounds__(kBlock, OT_LSE_WAVES_PER_SIMD) void lse_gather_kernel(
     const float *__restrict__ logits, const int32_t *__restrict__ targets,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
-    int N, int targets_cols, int64_t rows, int V, int blank, int rows_per_block,
-    float *__restrict__ den, float *__restrict__ lp) {
+    int N, int targets_cols, int64_t row_begin, int64_t rows, int V, int blank,
+    int rows_per_block, float *__restrict__ den, float *__restrict__ lp) {
   constexpr int G = kWave / L;
   constexpr bool kStaged = G > 1;
   __shared__ BlockUtterances bu;
   __shared__ __attribute__((aligned(16))) float s_stage[kStaged ? kWavesPerBlock * kWave * K * VEC : 4];
-  const int64_t row_first = (int64_t)blockIdx.x * rows_per_block;
+  // this launch covers rows [row_begin, rows)
+  const int64_t row_first = row_begin + (int64_t)blockIdx.x * rows_per_block;
   const int64_t row_end = min(rows, row_first + rows_per_block);
   bu.load(row_splits, N, row_first, row_end - 1);
   const int64_t lattice_rows = row_splits[N];
@@ -266,9 +273,10 @@ __global__ __launch_bounds__(kBlock, OT_LSE_WAVES_PER_SIMD) void lse_gather_kern
 __global__ __launch_bounds__(kBlock) void gather_kernel(
     const float *__restrict__ logits, const int32_t *__restrict__ targets,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
-    int N, int targets_cols, int64_t rows, int V, int blank, float *__restrict__ lp) {
+    int N, int targets_cols, int64_t row_begin, int64_t rows, int V, int blank,
+    float *__restrict__ lp) {
   __shared__ BlockUtterances bu;
-  const int64_t row_first = (int64_t)blockIdx.x * kBlock;
+  const int64_t row_first = row_begin + (int64_t)blockIdx.x * kBlock;
   const int64_t row_end = min(rows, row_first + kBlock);
   bu.load(row_splits, N, row_first, row_end - 1);
   const int64_t row = row_first + threadIdx.x;
@@ -329,7 +337,8 @@ __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int 
 
   // This utterance's slice as raw buffers: a cell index outside [0, T*U1)
   // (t < 0, t >= T, or the forced offset of a thread without a column) reads
-  // as 0 and is not written.
+  // as 0 and is not written.  Byte offsets are carried directly; the high bit
+  // that pushes a column-less thread out of range survives the 32-bit adds.
   const unsigned cells = (unsigned)T * (unsigned)U1;
   const __amdgpu_buffer_rsrc_t lp_buf = make_buffer(lp + 2 * row0, cells * 8u);
   const __amdgpu_buffer_rsrc_t out_buf = make_buffer(out + row0, cells * 4u);
@@ -337,31 +346,40 @@ __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int 
   const int dt = BETA ? -1 : 1;
   const int dcell = BETA ? -U1 : U1;
   int t = BETA ? (T - 1 + delay) : -delay;  // lattice row at step 0
-  int cell = t * U1 + u;
+  const int cell0 = t * U1 + u;
+  unsigned off_out = (unsigned)cell0 * 4u + oob;                          // this step's cell
+  unsigned off_lp = (unsigned)(cell0 + kChunk * dcell) * 8u + oob;        // kChunk steps ahead
+  const unsigned d_out = (unsigned)dcell * 4u, d_lp = (unsigned)dcell * 8u;
 
-  auto fetch = [&](int c) -> f32x2 {
-    return __builtin_bit_cast(
-        f32x2, __builtin_amdgcn_raw_buffer_load_b64(lp_buf, ((unsigned)c * 8u) | oob, 0, 0));
+  auto fetch = [&](unsigned byte_off) -> f32x2 {
+    return __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(lp_buf, byte_off, 0, 0));
   };
 
   // wave whose edge lane feeds this wave, if any
   const int src_wave = BETA ? wave + 1 : wave - 1;
   const bool has_src = MULTI && src_wave >= 0 && src_wave <= wlast;
   const int edge_lane = BETA ? 0 : kWave - 1;
+  // where this lane's per-step ring write goes: the edge lane publishes, every
+  // other lane hits a dummy slot behind the ring
+  float *const ring_dst = &s_ring[wave][(lane == edge_lane) ? 0 : kRing];
+  const int ring_mask = (lane == edge_lane) ? (kRing - 1) : 0;
 
   // alpha: own = alpha(t-1,u)+blank(t-1,u), nb = alpha(t,u)+sym(t,u) handed to u+1
   // beta : own = nb = beta of the cell computed in the previous step
   // The lattice's start cell falls out of the recursion from own = 0:
   //   alpha(0,0) = log_add(0, -inf) = 0,  beta(T-1,U) = log_add(0 + blank, -inf) = blank.
+  // No step is masked: before a thread's first cell everything it sees is -inf
+  // (out-of-range lp reads give 0, and -inf + 0 = -inf), after its last cell its
+  // values only reach threads that are past their last cell too, and all stores
+  // outside the lattice are dropped by the buffer bounds.
   float own = (column && u == (BETA ? U : 0)) ? 0.f : OT_NEG_INF;
   float nb = OT_NEG_INF;
-  float fin = OT_NEG_INF;  // what the sweep hands out as the utterance's score
 
   // Ring of kChunk prefetched lp values: slot i is consumed at step n+i and
   // refilled at once for step n+i+kChunk.
   f32x2 q[kChunk];
 #pragma unroll
-  for (int i = 0; i < kChunk; ++i) q[i] = fetch(cell + i * dcell);
+  for (int i = 0; i < kChunk; ++i) q[i] = fetch((unsigned)(cell0 + i * dcell) * 8u + oob);
 
   for (int n = 0; n < nsteps; n += kChunk) {
     // the kChunk edge values of this chunk were all written before the last
@@ -374,8 +392,7 @@ __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int 
 #pragma unroll
     for (int i = 0; i < kChunk; ++i) {
       const f32x2 l = q[i];
-      q[i] = fetch(cell + kChunk * dcell);
-      const bool valid = column & ((unsigned)t < (unsigned)T);
+      q[i] = fetch(off_lp);
       float edge = OT_NEG_INF;
       if (MULTI)
         edge = __builtin_bit_cast(
@@ -383,38 +400,42 @@ __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int 
       const float in = BETA ? wave_shift_down(nb, edge) : wave_shift_up(nb, edge);
       float a = BETA ? OT_DP_LOG_ADD(own + l.x, in + l.y) : OT_DP_LOG_ADD(own, in);
       if (OSF) a = ((unsigned)(t - u) < band) ? a : OT_NEG_INF;
-      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, a), out_buf,
-                                            ((unsigned)cell * 4u) | oob, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, a), out_buf, off_out, 0, 0);
       if (BETA) {
-        own = nb = valid ? a : OT_NEG_INF;
-        fin = valid ? a : fin;
+        own = nb = a;
       } else {
-        own = valid ? a + l.x : OT_NEG_INF;
-        nb = valid ? a + l.y : OT_NEG_INF;
-        fin = valid ? own : fin;
+        own = a + l.x;
+        nb = a + l.y;
       }
-      if (MULTI) {
-        // the edge lane publishes nb; every other lane writes a dummy slot
-        float *dst = &s_ring[wave][(lane == edge_lane) ? ((n + i) & (kRing - 1)) : kRing];
-        *dst = nb;
-      }
-      t += dt;
-      cell += dcell;
+      if (MULTI) ring_dst[(n + i) & ring_mask] = nb;
+      if (OSF) t += dt;
+      off_out += d_out;
+      off_lp += d_lp;
     }
-    if (MULTI) __syncthreads();
+    if (MULTI) lds_barrier();
   }
-  // alpha: alpha(T-1,U) + blank(T-1,U);  beta: beta(0,0)
-  if (column && u == (BETA ? 0 : U)) *score = fin;
+
+  // The utterance's score is read back from what this thread stored itself
+  // (alpha: thread U's alpha(T-1,U) plus blank(T-1,U); beta: thread 0's beta(0,0)).
+  if (column && u == (BETA ? 0 : U)) {
+    __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have completed
+    if (BETA) {
+      *score = out[row0];
+    } else {
+      const int64_t last = row0 + (int64_t)cells - 1;
+      *score = out[last] + lp[2 * last];
+    }
+  }
 }
 
 template <bool OSF, bool MULTI>
 __global__ __launch_bounds__(OT_MAX_U1) void alpha_beta_kernel(
     const float *__restrict__ lp, const int32_t *__restrict__ logit_lengths,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
-    float *__restrict__ alpha, float *__restrict__ beta, float *__restrict__ scores_alpha,
-    float *__restrict__ scores_beta) {
+    int utt_begin, float *__restrict__ alpha, float *__restrict__ beta,
+    float *__restrict__ scores_alpha, float *__restrict__ scores_beta) {
   __shared__ float s_ring[MULTI ? kMaxDpWaves : 1][kRing + 1];
-  const int b = blockIdx.x;
+  const int b = utt_begin + blockIdx.x;
   const int T = logit_lengths[b], U = target_lengths[b];
   const int64_t row0 = row_splits[b];
   if (blockIdx.y == 0)
@@ -448,10 +469,10 @@ __global__ __launch_bounds__(kBlock) void row_coeff_kernel(
     const float *__restrict__ alpha, const float *__restrict__ beta,
     const int32_t *__restrict__ targets, const int32_t *__restrict__ logit_lengths,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits, int N,
-    int targets_cols, int64_t rows, int blank, int osf, float scale,
+    int targets_cols, int64_t row_begin, int64_t rows, int blank, int osf, float scale,
     float4 *__restrict__ coef_f, int2 *__restrict__ coef_i) {
   __shared__ BlockUtterances bu;
-  const int64_t row_first = (int64_t)blockIdx.x * kBlock;
+  const int64_t row_first = row_begin + (int64_t)blockIdx.x * kBlock;
   const int64_t row_end = min(rows, row_first + kBlock);
   bu.load(row_splits, N, row_first, row_end - 1);
   const int64_t row = row_first + threadIdx.x;
@@ -508,8 +529,10 @@ constexpr int kGradUnroll = 4;
 template <int VEC, bool FLS>
 __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
     const float *logits, float *grad, const float4 *__restrict__ coef_f,
-    const int2 *__restrict__ coef_i, int64_t nunits, int nvec, float inv_nvec, float scale) {
-  const int64_t base = (int64_t)blockIdx.x * (kGradUnroll * kBlock);
+    const int2 *__restrict__ coef_i, int64_t unit_begin, int64_t nunits, int nvec, float inv_nvec,
+    float scale) {
+  // this launch covers units [unit_begin, nunits)
+  const int64_t base = unit_begin + (int64_t)blockIdx.x * (kGradUnroll * kBlock);
   const int64_t row_base = base / nvec;
   const int rem_base = (int)(base - row_base * nvec);
   // the workgroup's units as raw buffers: the tail of the last workgroup needs no branch
@@ -659,13 +682,14 @@ extern "C" {
 
 int ot_row_splits(const int32_t *logit_lengths, const int32_t *target_lengths,
                   const int32_t *targets, int32_t N, int32_t targets_cols, int32_t *row_splits,
-                  ot_batch_status *status, void *stream) {
+                  int32_t *row_splits_mirror, ot_batch_status *status, void *stream) {
   if (!logit_lengths || !target_lengths || !row_splits || !status || N <= 0 || targets_cols < 0 ||
       (targets_cols > 0 && !targets))
     return OT_E_BAD_ARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipLaunchKernelGGL(prepare_kernel, dim3(1), dim3(kPrepThreads), 0, s, logit_lengths,
-                     target_lengths, targets, N, targets_cols, row_splits, status);
+                     target_lengths, targets, N, targets_cols, row_splits, row_splits_mirror,
+                     status);
   return launch_status();
 }
 
@@ -679,44 +703,59 @@ int ot_row_ids(const int32_t *row_splits, int32_t N, int64_t rows, int32_t *row_
   return launch_status();
 }
 
+int ot_log_probs_range(const float *logits, const int32_t *targets, const int32_t *target_lengths,
+                       const int32_t *row_splits, int32_t N, int32_t targets_cols, int64_t rows,
+                       int32_t V, int32_t blank, int32_t from_log_softmax, int64_t row_begin,
+                       int64_t row_end, float *den, float *lp, void *stream) {
+  if (!logits || !target_lengths || !row_splits || !lp || N <= 0 || rows <= 0 ||
+      rows > INT32_MAX || V <= 0 || blank < 0 || blank >= V || targets_cols < 0 ||
+      (targets_cols > 0 && !targets) || (!from_log_softmax && !den) || row_begin < 0 ||
+      row_end > rows || row_begin > row_end)
+    return OT_E_BAD_ARG;
+  if (reinterpret_cast<uintptr_t>(logits) & 3) return OT_E_MISALIGNED;
+  if (row_begin == row_end) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t count = row_end - row_begin;
+  if (from_log_softmax) {
+    const unsigned blocks = (unsigned)((count + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(kBlock), 0, s, logits, targets,
+                       target_lengths, row_splits, N, targets_cols, row_begin, row_end, V, blank,
+                       lp);
+    return launch_status();
+  }
+  const RowTiling t = pick_tiling(V, is_aligned16(logits));
+  const dim3 grid((unsigned)((count + t.rows_per_block - 1) / t.rows_per_block));
+  OT_DISPATCH(lse_gather_kernel, t, logits, targets, target_lengths, row_splits, N, targets_cols,
+              row_begin, row_end, V, blank, t.rows_per_block, den, lp)
+  return launch_status();
+}
+
 int ot_log_probs(const float *logits, const int32_t *targets, const int32_t *target_lengths,
                  const int32_t *row_splits, int32_t N, int32_t targets_cols, int64_t rows,
                  int32_t V, int32_t blank, int32_t from_log_softmax, float *den, float *lp,
                  void *stream) {
-  if (!logits || !target_lengths || !row_splits || !lp || N <= 0 || rows <= 0 ||
-      rows > INT32_MAX || V <= 0 || blank < 0 || blank >= V || targets_cols < 0 ||
-      (targets_cols > 0 && !targets) || (!from_log_softmax && !den))
-    return OT_E_BAD_ARG;
-  if (reinterpret_cast<uintptr_t>(logits) & 3) return OT_E_MISALIGNED;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (from_log_softmax) {
-    const unsigned blocks = (unsigned)((rows + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(kBlock), 0, s, logits, targets,
-                       target_lengths, row_splits, N, targets_cols, rows, V, blank, lp);
-    return launch_status();
-  }
-  const RowTiling t = pick_tiling(V, is_aligned16(logits));
-  const dim3 grid((unsigned)((rows + t.rows_per_block - 1) / t.rows_per_block));
-  OT_DISPATCH(lse_gather_kernel, t, logits, targets, target_lengths, row_splits, N, targets_cols,
-              rows, V, blank, t.rows_per_block, den, lp)
-  return launch_status();
+  return ot_log_probs_range(logits, targets, target_lengths, row_splits, N, targets_cols, rows, V,
+                            blank, from_log_softmax, 0, rows, den, lp, stream);
 }
 
-int ot_alpha_beta(const float *lp, const int32_t *logit_lengths, const int32_t *target_lengths,
-                  const int32_t *row_splits, int32_t N, int32_t max_u1, int32_t one_sym_per_frame,
-                  float *alpha, float *beta, float *scores_alpha, float *scores_beta,
-                  void *stream) {
+int ot_alpha_beta_range(const float *lp, const int32_t *logit_lengths,
+                        const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
+                        int32_t max_u1, int32_t one_sym_per_frame, int32_t utt_begin,
+                        int32_t utt_end, float *alpha, float *beta, float *scores_alpha,
+                        float *scores_beta, void *stream) {
   if (!lp || !logit_lengths || !target_lengths || !row_splits || !alpha || !beta ||
-      !scores_alpha || !scores_beta || N <= 0 || max_u1 <= 0)
+      !scores_alpha || !scores_beta || N <= 0 || max_u1 <= 0 || utt_begin < 0 || utt_end > N ||
+      utt_begin > utt_end)
     return OT_E_BAD_ARG;
   if (max_u1 > OT_MAX_U1) return OT_E_TOO_LONG;
+  if (utt_begin == utt_end) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int threads = ((max_u1 + kWave - 1) / kWave) * kWave;
-  const dim3 grid((unsigned)N, 2), block((unsigned)threads);
+  const dim3 grid((unsigned)(utt_end - utt_begin), 2), block((unsigned)threads);
   const bool multi = threads > kWave;
 #define OT_LAUNCH_DP(OSF_, MULTI_)                                                              \
   hipLaunchKernelGGL((alpha_beta_kernel<OSF_, MULTI_>), grid, block, 0, s, lp, logit_lengths,   \
-                     target_lengths, row_splits, alpha, beta, scores_alpha, scores_beta)
+                     target_lengths, row_splits, utt_begin, alpha, beta, scores_alpha, scores_beta)
   if (one_sym_per_frame) {
     if (multi) OT_LAUNCH_DP(true, true); else OT_LAUNCH_DP(true, false);
   } else {
@@ -726,54 +765,81 @@ int ot_alpha_beta(const float *lp, const int32_t *logit_lengths, const int32_t *
   return launch_status();
 }
 
+int ot_alpha_beta(const float *lp, const int32_t *logit_lengths, const int32_t *target_lengths,
+                  const int32_t *row_splits, int32_t N, int32_t max_u1, int32_t one_sym_per_frame,
+                  float *alpha, float *beta, float *scores_alpha, float *scores_beta,
+                  void *stream) {
+  return ot_alpha_beta_range(lp, logit_lengths, target_lengths, row_splits, N, max_u1,
+                             one_sym_per_frame, 0, N, alpha, beta, scores_alpha, scores_beta,
+                             stream);
+}
+
+int ot_row_coefficients_range(const float *lp, const float *den, const float *alpha,
+                              const float *beta, const int32_t *targets,
+                              const int32_t *logit_lengths, const int32_t *target_lengths,
+                              const int32_t *row_splits, int32_t N, int32_t targets_cols,
+                              int64_t rows, int32_t blank, int32_t from_log_softmax,
+                              int32_t one_sym_per_frame, float grad_scale, int64_t row_begin,
+                              int64_t row_end, void *row_scratch, void *stream) {
+  if (!alpha || !beta || !logit_lengths || !target_lengths || !row_splits || !row_scratch ||
+      N <= 0 || rows <= 0 || rows > INT32_MAX || blank < 0 || targets_cols < 0 ||
+      (targets_cols > 0 && !targets) || (from_log_softmax ? !lp : !den) || row_begin < 0 ||
+      row_end > rows || row_begin > row_end)
+    return OT_E_BAD_ARG;
+  if (reinterpret_cast<uintptr_t>(row_scratch) & 15) return OT_E_MISALIGNED;
+  if (row_begin == row_end) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float4 *coef_f = static_cast<float4 *>(row_scratch);
+  int2 *coef_i = reinterpret_cast<int2 *>(coef_f + rows);
+  const dim3 grid((unsigned)((row_end - row_begin + kBlock - 1) / kBlock));
+  if (from_log_softmax)
+    hipLaunchKernelGGL(row_coeff_kernel<true>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
+                       targets, logit_lengths, target_lengths, row_splits, N, targets_cols,
+                       row_begin, row_end, blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
+  else
+    hipLaunchKernelGGL(row_coeff_kernel<false>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
+                       targets, logit_lengths, target_lengths, row_splits, N, targets_cols,
+                       row_begin, row_end, blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
+  return launch_status();
+}
+
 int ot_row_coefficients(const float *lp, const float *den, const float *alpha, const float *beta,
                         const int32_t *targets, const int32_t *logit_lengths,
                         const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
                         int32_t targets_cols, int64_t rows, int32_t blank,
                         int32_t from_log_softmax, int32_t one_sym_per_frame, float grad_scale,
                         void *row_scratch, void *stream) {
-  if (!alpha || !beta || !logit_lengths || !target_lengths || !row_splits || !row_scratch ||
-      N <= 0 || rows <= 0 || rows > INT32_MAX || blank < 0 || targets_cols < 0 ||
-      (targets_cols > 0 && !targets) || (from_log_softmax ? !lp : !den))
-    return OT_E_BAD_ARG;
-  if (reinterpret_cast<uintptr_t>(row_scratch) & 15) return OT_E_MISALIGNED;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  float4 *coef_f = static_cast<float4 *>(row_scratch);
-  int2 *coef_i = reinterpret_cast<int2 *>(coef_f + rows);
-  const dim3 grid((unsigned)((rows + kBlock - 1) / kBlock));
-  if (from_log_softmax)
-    hipLaunchKernelGGL(row_coeff_kernel<true>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
-                       targets, logit_lengths, target_lengths, row_splits, N, targets_cols, rows,
-                       blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
-  else
-    hipLaunchKernelGGL(row_coeff_kernel<false>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
-                       targets, logit_lengths, target_lengths, row_splits, N, targets_cols, rows,
-                       blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
-  return launch_status();
+  return ot_row_coefficients_range(lp, den, alpha, beta, targets, logit_lengths, target_lengths,
+                                   row_splits, N, targets_cols, rows, blank, from_log_softmax,
+                                   one_sym_per_frame, grad_scale, 0, rows, row_scratch, stream);
 }
 
-int ot_gradient_apply(const float *logits, const void *row_scratch, int64_t rows, int32_t V,
-                      int32_t from_log_softmax, float grad_scale, float *grad, void *stream) {
-  if (!row_scratch || !grad || rows <= 0 || rows > INT32_MAX || V <= 0) return OT_E_BAD_ARG;
+int ot_gradient_apply_range(const float *logits, const void *row_scratch, int64_t rows, int32_t V,
+                            int32_t from_log_softmax, float grad_scale, int64_t row_begin,
+                            int64_t row_end, float *grad, void *stream) {
+  if (!row_scratch || !grad || rows <= 0 || rows > INT32_MAX || V <= 0 || row_begin < 0 ||
+      row_end > rows || row_begin > row_end)
+    return OT_E_BAD_ARG;
   if (from_log_softmax ? grad == logits : !logits) return OT_E_BAD_ARG;
   if ((reinterpret_cast<uintptr_t>(grad) & 3) || (reinterpret_cast<uintptr_t>(logits) & 3) ||
       (reinterpret_cast<uintptr_t>(row_scratch) & 15))
     return OT_E_MISALIGNED;
+  if (row_begin == row_end) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float4 *coef_f = static_cast<const float4 *>(row_scratch);
   const int2 *coef_i = reinterpret_cast<const int2 *>(coef_f + rows);
   const bool aligned = is_aligned16(grad) && (from_log_softmax || is_aligned16(logits));
   const int vec = (aligned && V % 4 == 0) ? 4 : 1;
   const int nvec = V / vec;
-  const int64_t nunits = rows * nvec;
+  const int64_t unit_begin = row_begin * nvec, unit_end = row_end * nvec;
   const int64_t per_block = (int64_t)kGradUnroll * kBlock;
-  const int64_t blocks = (nunits + per_block - 1) / per_block;
+  const int64_t blocks = (unit_end - unit_begin + per_block - 1) / per_block;
   if (blocks > INT32_MAX) return OT_E_BAD_ARG;
   const dim3 grid((unsigned)blocks);
   const float inv_nvec = 1.0f / (float)nvec;
 #define OT_LAUNCH_GRAD(VEC_, FLS_)                                                            \
   hipLaunchKernelGGL((grad_flat_kernel<VEC_, FLS_>), grid, dim3(kBlock), 0, s, logits, grad,  \
-                     coef_f, coef_i, nunits, nvec, inv_nvec, grad_scale)
+                     coef_f, coef_i, unit_begin, unit_end, nvec, inv_nvec, grad_scale)
   if (from_log_softmax) {
     if (vec == 4) OT_LAUNCH_GRAD(4, true); else OT_LAUNCH_GRAD(1, true);
   } else {
@@ -781,6 +847,12 @@ int ot_gradient_apply(const float *logits, const void *row_scratch, int64_t rows
   }
 #undef OT_LAUNCH_GRAD
   return launch_status();
+}
+
+int ot_gradient_apply(const float *logits, const void *row_scratch, int64_t rows, int32_t V,
+                      int32_t from_log_softmax, float grad_scale, float *grad, void *stream) {
+  return ot_gradient_apply_range(logits, row_scratch, rows, V, from_log_softmax, grad_scale, 0,
+                                 rows, grad, stream);
 }
 
 int ot_gradient(const float *logits, const float *lp, const float *den, const float *alpha,
@@ -845,7 +917,7 @@ int ot_transducer_loss(const float *logits, const int32_t *targets, const int32_
   float *beta = reinterpret_cast<float *>(w);           w += align256((size_t)rows * sizeof(float));
   void *row_scratch = w;
   int rc = ot_row_splits(logit_lengths, target_lengths, targets, N, targets_cols, row_splits,
-                         status, stream);
+                         nullptr, status, stream);
   if (rc) return rc;
   rc = ot_log_probs(logits, targets, target_lengths, row_splits, N, targets_cols, rows, V, blank,
                     from_log_softmax, den, lp, stream);

@@ -50,7 +50,7 @@ def row_splits(T, U, targets):
     status = torch.zeros(ctypes.sizeof(BatchStatus), dtype=torch.uint8, device=T.device)
     cols = targets.shape[1]
     check(lib().ot_row_splits(ptr(T), ptr(U), ptr(targets if cols else None), ctypes.c_int32(N),
-                              ctypes.c_int32(cols), ptr(splits), ptr(status), stream()))
+                              ctypes.c_int32(cols), ptr(splits), ptr(None), ptr(status), stream()))
     st = BatchStatus.from_buffer_copy(status.cpu().numpy().tobytes())
     return splits, st
 

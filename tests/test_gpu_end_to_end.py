@@ -195,6 +195,28 @@ def test_reference_test_shapes_modified_logits_vs_logsoftmax(device):
     assert np.allclose(a.grad.cpu().numpy(), want, atol=1e-4)
 
 
+def test_two_stream_schedule_gives_the_same_bits(device):
+    # opt-in schedule: lattice kernel of one half of the batch on a second stream
+    import optimized_transducer_amd as ot
+    ext = ot._optimized_transducer
+    w = workloads.asr_batch(N=8, V=512, scale=0.8)  # above the size threshold of the schedule
+    x = w.logits_torch(device)
+    tg, T, U = _dev(w.targets, device), _dev(w.logit_lengths, device), _dev(w.target_lengths, device)
+    out = []
+    for on in (False, True, False):
+        ext.set_overlap(on)
+        try:
+            logits = x.clone().requires_grad_(True)
+            loss = ot.transducer_loss(logits, tg, T, U, 0, False, reduction="mean")
+            loss.backward()
+            torch.cuda.synchronize()
+            out.append((loss.detach().clone(), logits.grad.clone()))
+        finally:
+            ext.set_overlap(False)
+    for loss, grad in out[1:]:
+        assert torch.equal(loss, out[0][0]) and torch.equal(grad, out[0][1])
+
+
 # ------------------------------------------------------------------ full sizes
 FULL = [
     ("asr", lambda: workloads.asr_batch()),

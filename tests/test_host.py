@@ -38,7 +38,7 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_device():
     L = cabi.lib()
     null = ctypes.c_void_p(0)
     i32, i64 = ctypes.c_int32, ctypes.c_int64
-    assert L.ot_row_splits(null, null, null, i32(4), i32(3), null, null, null) == -1
+    assert L.ot_row_splits(null, null, null, i32(4), i32(3), null, null, null, null) == -1
     assert L.ot_row_ids(null, i32(1), i64(5), null, null) == -1
     assert L.ot_log_probs(null, null, null, null, i32(1), i32(0), i64(4), i32(8), i32(0), i32(0),
                           null, null, null) == -1
