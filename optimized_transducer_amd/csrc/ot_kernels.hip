@@ -80,9 +80,22 @@ __global__ __launch_bounds__(kPrepThreads) void prepare_kernel(
     umax = max(umax, U); umin = min(umin, U);
     tmax = max(tmax, T); tmin = min(tmin, T);
   }
+  // min/max over all N * targets_cols entries: 16-byte loads, several in flight per thread
   int gmax = INT32_MIN, gmin = INT32_MAX;
   const long long ntargets = (long long)N * targets_cols;
-  for (long long i = tid; i < ntargets; i += kPrepThreads) {
+  long long done = 0;
+  if ((reinterpret_cast<uintptr_t>(targets) & 15) == 0) {
+    const int4 *t4 = reinterpret_cast<const int4 *>(targets);
+    const long long n4 = ntargets / 4;
+#pragma unroll 4
+    for (long long i = tid; i < n4; i += kPrepThreads) {
+      const int4 v = t4[i];
+      gmax = max(max(gmax, v.x), max(max(v.y, v.z), v.w));
+      gmin = min(min(gmin, v.x), min(min(v.y, v.z), v.w));
+    }
+    done = n4 * 4;
+  }
+  for (long long i = done + tid; i < ntargets; i += kPrepThreads) {
     const int v = targets[i];
     gmax = max(gmax, v); gmin = min(gmin, v);
   }
