@@ -81,24 +81,14 @@ __device__ __forceinline__ float exp_fast(float x) {
   return __builtin_amdgcn_exp2f(x * 1.44269502162933349609375f);
 }
 
-// exp(x) for x <= 0 through the hardware 2^x unit.  The product x*log2(e) is
-// formed in two pieces (rounded product + its exact residual) so that the
-// argument error does not grow with |x|; result within about 1 ulp.
-__device__ __forceinline__ float exp_neg(float x) {
-  constexpr float kLog2eHi = 1.44269502162933349609375f;      // float(log2(e))
-  constexpr float kLog2eLo = 1.92596299112661746e-8f;         // log2(e) - kLog2eHi
-  constexpr float kLn2 = 0.693147182464599609375f;
-  const float ph = x * kLog2eHi;
-  const float pl = __builtin_fmaf(x, kLog2eHi, -ph) + x * kLog2eLo;
-  const float e = __builtin_amdgcn_exp2f(ph);
-  return __builtin_fmaf(e, pl * kLn2, e);
-}
-
-// exp(x) for any x: same evaluation, with the limits (0, +inf) passed through
-// so that x = -inf (a masked logit) gives exactly 0.
+// exp(x) for any x through the hardware 2^x unit, accurate to about 1 ulp:
+// the product x*log2(e) is formed in two pieces (rounded product + its exact
+// residual) so that the argument error does not grow with |x|.  The limits
+// (0, +inf) are passed through, so x = -inf (a masked logit) gives exactly 0.
+// Used for the gradient entries.
 __device__ __forceinline__ float exp_any(float x) {
-  constexpr float kLog2eHi = 1.44269502162933349609375f;
-  constexpr float kLog2eLo = 1.92596299112661746e-8f;
+  constexpr float kLog2eHi = 1.44269502162933349609375f;  // float(log2(e))
+  constexpr float kLog2eLo = 1.92596299112661746e-8f;     // log2(e) - kLog2eHi
   constexpr float kLn2 = 0.693147182464599609375f;
   const float ph = x * kLog2eHi;
   const float pl = __builtin_fmaf(x, kLog2eHi, -ph) + x * kLog2eLo;
@@ -107,31 +97,14 @@ __device__ __forceinline__ float exp_any(float x) {
   return (e == 0.0f || __builtin_isinf(e)) ? e : r;
 }
 
-// log1p(e) for e in [0, 1]: hardware log2 of u = 1 + e, plus the first-order
-// correction for the rounding of u.
-__device__ __forceinline__ float log1p_unit(float e) {
-  constexpr float kLn2 = 0.693147182464599609375f;
-  const float u = 1.0f + e;
-  const float l = __builtin_amdgcn_logf(u) * kLn2;
-  return l + (e - (u - 1.0f)) * __builtin_amdgcn_rcpf(u);
-}
-
 // log(exp(a) + exp(b)) ordered as the reference's CPU LogSumExp (cpu.cc:18-35):
 // larger + log1p(exp(smaller - larger)), or just the larger one when the
-// difference is below kMinLogDiff or is NaN (-inf minus -inf).
+// difference is below kMinLogDiff or is NaN (-inf minus -inf).  Both
+// transcendental steps run straight on the hardware units (2^x and log2);
+// absolute error of the added term about 1.5e-7, i.e. below one ulp of the
+// result as soon as |larger| >= 2.  This function is the critical path of the
+// lattice sweep.
 __device__ __forceinline__ float log_add(float a, float b) {
-  const bool lt = a < b;
-  const float hi = lt ? b : a;
-  const float diff = lt ? (a - b) : (b - a);
-  const float add = (diff >= kMinLogDiff) ? log1p_unit(exp_neg(diff)) : 0.0f;
-  return hi + add;
-}
-
-// Same ordering, both transcendental steps straight on the hardware units
-// (2^x and log2).  Absolute error of the added term about 1.5e-7, i.e. below
-// one ulp of the result as soon as |larger| >= 2; used by the lattice sweep,
-// whose critical path is this function.
-__device__ __forceinline__ float log_add_fast(float a, float b) {
   constexpr float kLog2e = 1.44269502162933349609375f;
   constexpr float kLn2 = 0.693147182464599609375f;
   // smaller - larger = -|a - b| (the sign and abs fold into operand modifiers);
@@ -228,10 +201,7 @@ __device__ __forceinline__ Cell decode_row(const BlockUtterances &bu, int64_t ro
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 // cache-policy operand of the raw buffer builtins: bit 1 = non-temporal
-#ifndef OT_AUX_STREAM
-#define OT_AUX_STREAM 2
-#endif
-constexpr int kAuxStream = OT_AUX_STREAM;
+constexpr int kAuxStream = 2;
 
 // VEC floats of a row.  The (rows, V) arrays are streamed once per kernel and
 // never re-read by the same kernel, so their loads and stores carry the
@@ -240,11 +210,7 @@ template <int VEC> struct Vec;
 template <> struct Vec<4> {
   float v[4];
   __device__ __forceinline__ void load(const float *p) {
-#ifdef OT_NO_NT_LOAD
-    const f32x4 x = *reinterpret_cast<const f32x4 *>(p);
-#else
     const f32x4 x = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
-#endif
     v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
   }
   __device__ __forceinline__ void store(float *p) const {
@@ -269,11 +235,7 @@ template <> struct Vec<4> {
   // cache line is much slower than a cached one
   __device__ __forceinline__ void store_stream(float *p) const {
     const f32x4 x = {v[0], v[1], v[2], v[3]};
-#ifdef OT_NO_NT_STORE
-    *reinterpret_cast<f32x4 *>(p) = x;
-#else
     __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(p));
-#endif
   }
 };
 template <> struct Vec<1> {

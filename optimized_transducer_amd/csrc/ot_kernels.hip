@@ -142,11 +142,8 @@ __global__ void row_ids_kernel(const int32_t *__restrict__ row_splits, int N, in
 // current pass is reduced.  The blank/target gather then reads LDS, not HBM.
 // Rows longer than L*K vectors (L = 64, so flat and row-group layout coincide)
 // stream through registers in chunks with a running (max, scaled sum).
-#ifndef OT_LSE_WAVES_PER_SIMD
-#define OT_LSE_WAVES_PER_SIMD 1
-#endif
 template <int VEC, int L, int K>
-__global__ __launch_bounds__(kBlock, OT_LSE_WAVES_PER_SIMD) void lse_gather_kernel(
+__global__ __launch_bounds__(kBlock) void lse_gather_kernel(
     const float *__restrict__ logits, const int32_t *__restrict__ targets,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
     int N, int targets_cols, int64_t row_begin, int64_t rows, int V, int blank,
@@ -325,9 +322,6 @@ constexpr int kChunk = 16;  // steps between barriers
 constexpr int kLag = kChunk;
 constexpr int kRing = 64;   // >= 2*kChunk + 2 slots per wave boundary
 
-#ifndef OT_DP_LOG_ADD
-#define OT_DP_LOG_ADD log_add_fast
-#endif
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 template <bool BETA, bool OSF, bool MULTI>
@@ -411,7 +405,7 @@ __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int 
         edge = __builtin_bit_cast(
             float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ering), i));
       const float in = BETA ? wave_shift_down(nb, edge) : wave_shift_up(nb, edge);
-      float a = BETA ? OT_DP_LOG_ADD(own + l.x, in + l.y) : OT_DP_LOG_ADD(own, in);
+      float a = BETA ? log_add(own + l.x, in + l.y) : log_add(own, in);
       if (OSF) a = ((unsigned)(t - u) < band) ? a : OT_NEG_INF;
       __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, a), out_buf, off_out, 0, 0);
       if (BETA) {
@@ -472,9 +466,6 @@ __global__ __launch_bounds__(OT_MAX_U1) void alpha_beta_kernel(
 // column when a target equals blank.  col1 == kZeroRow marks an all-zero row
 // (outside the one-symbol-per-frame band, or likelihood not finite).
 constexpr int kZeroRow = -2;
-#ifndef OT_GRAD_EXP
-#define OT_GRAD_EXP exp_any
-#endif
 
 template <bool FLS>
 __global__ __launch_bounds__(kBlock) void row_coeff_kernel(
@@ -521,8 +512,8 @@ __global__ __launch_bounds__(kBlock) void row_coeff_kernel(
       ci = make_int2(col1, col2);
       if (FLS) {
         const float2 l = reinterpret_cast<const float2 *>(lp)[row];
-        f.x = col1 >= 0 ? -OT_GRAD_EXP((l.x + cc) + e1) * scale : 0.f;
-        f.y = col2 >= 0 ? -OT_GRAD_EXP((l.y + cc) + e2) * scale : 0.f;
+        f.x = col1 >= 0 ? -exp_any((l.x + cc) + e1) * scale : 0.f;
+        f.y = col2 >= 0 ? -exp_any((l.y + cc) + e2) * scale : 0.f;
       } else {
         f = make_float4(cc, bt, e1, e2);
       }
@@ -536,17 +527,24 @@ __global__ __launch_bounds__(kBlock) void row_coeff_kernel(
 // row i / nvec.  Consecutive lanes touch consecutive 16-byte units, so every
 // wave instruction moves one aligned, contiguous 1 KiB whatever V is; a
 // workgroup owns kGradUnroll * 256 consecutive units and exists only for them
-// (one-shot grid: the measured optimum for a read-modify-write stream here).
-constexpr int kGradUnroll = 4;
+// (one-shot grid, non-temporal accesses: the measured optimum here both for the
+// read-modify-write stream of the logits input and for the write-only stream
+// of the log-softmax input).
+constexpr int kGradUnroll = 2;  // 2 x 16 bytes per thread: fastest of 1, 2, 4, 8 on MI355X
 
 template <int VEC, bool FLS>
 __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
     const float *logits, float *grad, const float4 *__restrict__ coef_f,
     const int2 *__restrict__ coef_i, int64_t unit_begin, int64_t nunits, int nvec, float inv_nvec,
-    float scale) {
+    double inv_nvec_d, float scale) {
   // this launch covers units [unit_begin, nunits)
   const int64_t base = unit_begin + (int64_t)blockIdx.x * (kGradUnroll * kBlock);
-  const int64_t row_base = base / nvec;
+  // base / nvec through a double reciprocal (exact below 2^53) and one correction step
+  int64_t row_base = (int64_t)((double)base * inv_nvec_d);
+  {
+    const int64_t r = base - row_base * nvec;
+    if (r < 0) --row_base; else if (r >= nvec) ++row_base;
+  }
   const int rem_base = (int)(base - row_base * nvec);
   // the workgroup's units as raw buffers: the tail of the last workgroup needs no branch
   const unsigned span_bytes =
@@ -560,7 +558,7 @@ __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
   for (int k = 0; k < kGradUnroll; ++k) {
     const int local = k * kBlock + (int)threadIdx.x;
     if (!FLS) x[k].load_buffer(in_buf, (unsigned)local * (VEC * 4u));
-    // idx < nvec + 1024 is exact in float; one correction step fixes the quotient
+    // idx < nvec + kGradUnroll*256 is exact in float; one correction step fixes the quotient
     const int idx = rem_base + local;
     int q = (int)((float)idx * inv_nvec);
     if (q * nvec > idx) --q; else if ((q + 1) * nvec <= idx) ++q;
@@ -589,13 +587,13 @@ __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
     } else {
       const bool zero = ci.x == kZeroRow;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) y.v[e] = zero ? 0.f : OT_GRAD_EXP((x[k].v[e] + f.x) + f.y);
+      for (int e = 0; e < VEC; ++e) y.v[e] = zero ? 0.f : exp_any((x[k].v[e] + f.x) + f.y);
       const unsigned d1 = (unsigned)(ci.x - col0[k]), d2 = (unsigned)(ci.y - col0[k]);
       if (d1 < (unsigned)VEC || d2 < (unsigned)VEC) {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-          if (d1 == (unsigned)e) y.v[e] -= OT_GRAD_EXP((x[k].v[e] + f.x) + f.z);
-          if (d2 == (unsigned)e) y.v[e] -= OT_GRAD_EXP((x[k].v[e] + f.x) + f.w);
+          if (d1 == (unsigned)e) y.v[e] -= exp_any((x[k].v[e] + f.x) + f.z);
+          if (d2 == (unsigned)e) y.v[e] -= exp_any((x[k].v[e] + f.x) + f.w);
         }
       }
       if (scale != 1.f) {
@@ -637,9 +635,8 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const float4 *__restrict__
 // ---------------------------------------------------------------------------
 // host side: geometry and dispatch
 // ---------------------------------------------------------------------------
-#ifndef OT_TUNE_BLOCK_BYTES
-#define OT_TUNE_BLOCK_BYTES (256 * 1024)
-#endif
+// logits bytes one workgroup of the denominator kernel covers
+constexpr int64_t kLseBlockBytes = 256 * 1024;
 struct RowTiling {
   int vec, L, K, rows_per_block;
 };
@@ -657,7 +654,7 @@ static RowTiling pick_tiling(int V, bool aligned16) {
   t.K = K;
   // about 256 KiB of logits per workgroup, a whole number of wave passes
   const int pass = kWavesPerBlock * (kWave / L);
-  int64_t want = (OT_TUNE_BLOCK_BYTES) / ((int64_t)V * 4);
+  int64_t want = kLseBlockBytes / ((int64_t)V * 4);
   int rpb = (int)((want / pass) * pass);
   if (rpb < pass) rpb = pass;
   if (rpb > kMaxRowsPerBlock) rpb = kMaxRowsPerBlock;
@@ -852,7 +849,8 @@ int ot_gradient_apply_range(const float *logits, const void *row_scratch, int64_
   const float inv_nvec = 1.0f / (float)nvec;
 #define OT_LAUNCH_GRAD(VEC_, FLS_)                                                            \
   hipLaunchKernelGGL((grad_flat_kernel<VEC_, FLS_>), grid, dim3(kBlock), 0, s, logits, grad,  \
-                     coef_f, coef_i, unit_begin, unit_end, nvec, inv_nvec, grad_scale)
+                     coef_f, coef_i, unit_begin, unit_end, nvec, inv_nvec, 1.0 / (double)nvec,       \
+                     grad_scale)
   if (from_log_softmax) {
     if (vec == 4) OT_LAUNCH_GRAD(4, true); else OT_LAUNCH_GRAD(1, true);
   } else {
