@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # WRITE_SIZE runs scaled by the library's 1 GiB copy kernel (x2.000 / x1.000);
 # summary and commands in profiles/hbm_traffic_bench_asr_N32_V500.md.  Valid for
 # this workload and the kernel's current access pattern only.
-MEASURED_TRAFFIC_BYTES = {("asr_N32_V500", "grad_logits"): 3.0495e9}
+MEASURED_TRAFFIC_BYTES = {("asr_N32_V500", "grad_logits"): 3.0727e9}
 
 
 def make_workload(name):
