@@ -110,6 +110,11 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="asr")
+    ap.add_argument("--defer-gradient", action="store_true",
+                    help="use the deferred mode of the Python API (gradient pass in backward)")
+    ap.add_argument("--loss-weight", type=float, default=1.0,
+                    help="multiply the loss by this before backward (a weighted or scaled loss); "
+                         "the headline figure uses 1")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -139,7 +144,10 @@ def main():
     def step(buf):
         buf.requires_grad_(True)
         loss = ot.transducer_loss(buf, targets, T, U, w.blank, w.from_log_softmax,
-                                  w.one_sym_per_frame, w.reduction)
+                                  w.one_sym_per_frame, w.reduction,
+                                  defer_gradient=args.defer_gradient)
+        if args.loss_weight != 1.0:
+            loss = loss * args.loss_weight
         loss.backward()
         return loss
 
@@ -179,6 +187,9 @@ def main():
                    "one_sym_per_frame": w.one_sym_per_frame, "reduction": w.reduction,
                    "logits_bytes": 4 * w.rows * w.V, "seed": w.seed},
     }
+    if args.defer_gradient or args.loss_weight != 1.0:
+        out["config"]["defer_gradient"] = args.defer_gradient
+        out["config"]["loss_weight"] = args.loss_weight
 
     if not args.no_roofline:
         # second pass, per-kernel hipEvent timing on the launch stream

@@ -174,6 +174,19 @@ int ot_gradient_apply_range(const float *logits, const void *row_scratch,
                             float grad_scale, int64_t row_begin, int64_t row_end,
                             float *grad, void *stream);
 
+/* ot_gradient_apply with one more factor, read from DEVICE memory when the
+ * kernel runs: grad = d(-log-likelihood)/d(logits) * grad_scale * *device_factor.
+ * For a caller that postpones the (rows, V) pass until the upstream gradient
+ * of the loss is known (it keeps `row_scratch` and, for logits input, the
+ * logits themselves alive until then): this folds ctx.grad.mul_(loss_grad)
+ * (transducer_loss.py:162) into the one pass that writes the gradient, without
+ * the host ever reading loss_grad. */
+int ot_gradient_apply_device_factor(const float *logits, const void *row_scratch,
+                                    int64_t rows, int32_t V,
+                                    int32_t from_log_softmax, float grad_scale,
+                                    const float *device_factor, float *grad,
+                                    void *stream);
+
 /* Bytes of 16-byte aligned device scratch ot_gradient needs in `row_scratch`
  * (per-row coefficients, 24 bytes per packed row). */
 size_t ot_gradient_scratch_bytes(int64_t rows);

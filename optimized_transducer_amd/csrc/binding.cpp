@@ -139,10 +139,14 @@ void check_batch_values(const torch::Tensor &logits, const torch::Tensor &target
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// With `coefficients` set, the (rows, V) gradient pass is left to
+// apply_deferred_gradient: the per-row coefficients go into a tensor of their own,
+// handed back through the pointer, and the returned gradient is None.
 std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
     torch::Tensor &logits, const torch::Tensor &targets, const torch::Tensor &logit_lengths,
     const torch::Tensor &target_lengths, int32_t blank, bool from_log_softmax,
-    bool one_sym_per_frame, double grad_scale) {
+    bool one_sym_per_frame, double grad_scale, torch::Tensor *coefficients) {
+  const bool defer = coefficients != nullptr;
   auto logits_arg = torch::TensorArg(logits, "logits", 0);
   auto targets_arg = torch::TensorArg(targets, "targets", 1);
   auto logit_lengths_arg = torch::TensorArg(logit_lengths, "logit_lengths", 2);
@@ -203,10 +207,17 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   const size_t off_alpha = off_lp + align256(rows * 2 * sizeof(float));
   const size_t off_beta = off_alpha + align256(rows * sizeof(float));
   const size_t off_coef = off_beta + align256(rows * sizeof(float));
-  const size_t total = off_coef + align256(ot_gradient_scratch_bytes(rows));
+  const size_t total = off_coef + (defer ? 0 : align256(ot_gradient_scratch_bytes(rows)));
   torch::Tensor workspace =
       torch::empty({(int64_t)total}, logits.options().dtype(torch::kUInt8));
   char *w = static_cast<char *>(workspace.data_ptr());
+  char *coef = w + off_coef;
+  if (defer && logits.requires_grad()) {
+    // outlives this call, unlike the rest of the workspace
+    *coefficients = torch::empty({(int64_t)ot_gradient_scratch_bytes(rows)},
+                                 logits.options().dtype(torch::kUInt8));
+    coef = static_cast<char *>(coefficients->data_ptr());
+  }
   auto *row_splits = reinterpret_cast<int32_t *>(w);
   auto *scores_beta = reinterpret_cast<float *>(w + off_sbeta);
   auto *den = reinterpret_cast<float *>(w + off_den);
@@ -289,12 +300,12 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   torch::Tensor scores = torch::empty({N}, logits.options());
   torch::Tensor gradient;
   const bool want_grad = logits.requires_grad();
-  if (want_grad) {
+  if (want_grad && !defer) {
     // cpu.cc:803 / cuda.cu:444: new tensor for log-softmax input;
     // cpu.cc:814 / cuda.cu:449: the logits buffer itself otherwise.
     gradient = from_log_softmax ? torch::empty_like(logits) : logits;
   }
-  float *p_grad = want_grad ? gradient.data_ptr<float>() : nullptr;
+  float *p_grad = gradient.defined() ? gradient.data_ptr<float>() : nullptr;
 
   // lattice + per-row coefficients of utterances [b0, b1) on stream `s`
   auto lattice_part = [&](int32_t b0, int32_t b1, hipStream_t s) {
@@ -309,13 +320,13 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
       OT_CHECK(ot_row_coefficients_range(lp, den, alpha, beta, p_targets, p_T, p_U, row_splits,
                                          (int32_t)N, (int32_t)S, rows, blank, from_log_softmax,
                                          one_sym_per_frame, (float)grad_scale, splits_host[b0],
-                                         splits_host[b1], w + off_coef, s));
+                                         splits_host[b1], coef, s));
     }
   };
   auto gradient_part = [&](int32_t b0, int32_t b1) {
-    if (!want_grad) return;
+    if (!p_grad) return;
     ScopedTimer timer(from_log_softmax ? "grad_logsoftmax" : "grad_logits", stream);
-    OT_CHECK(ot_gradient_apply_range(p_logits, w + off_coef, rows, (int32_t)V, from_log_softmax,
+    OT_CHECK(ot_gradient_apply_range(p_logits, coef, rows, (int32_t)V, from_log_softmax,
                                      (float)grad_scale, splits_host[b0], splits_host[b1], p_grad,
                                      stream));
   };
@@ -356,7 +367,59 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_transducer_loss
     const torch::Tensor &target_lengths, int32_t blank, bool from_log_softmax,
     bool one_sym_per_frame) {
   return compute_impl(logits, targets, logit_lengths, target_lengths, blank, from_log_softmax,
-                      one_sym_per_frame, 1.0);
+                      one_sym_per_frame, 1.0, nullptr);
+}
+
+std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_transducer_loss_scaled(
+    torch::Tensor &logits, const torch::Tensor &targets, const torch::Tensor &logit_lengths,
+    const torch::Tensor &target_lengths, int32_t blank, bool from_log_softmax,
+    bool one_sym_per_frame, double grad_scale) {
+  return compute_impl(logits, targets, logit_lengths, target_lengths, blank, from_log_softmax,
+                      one_sym_per_frame, grad_scale, nullptr);
+}
+
+// Forward half of the deferred mode: everything but the (rows, V) pass.  Returns
+// (scores, per-row coefficients); the coefficients are None when logits does not
+// require grad.  Nothing is written to logits.
+std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_transducer_loss_deferred(
+    torch::Tensor &logits, const torch::Tensor &targets, const torch::Tensor &logit_lengths,
+    const torch::Tensor &target_lengths, int32_t blank, bool from_log_softmax,
+    bool one_sym_per_frame, double grad_scale) {
+  torch::Tensor coefficients;
+  auto out = compute_impl(logits, targets, logit_lengths, target_lengths, blank, from_log_softmax,
+                          one_sym_per_frame, grad_scale, &coefficients);
+  if (coefficients.defined()) return {out.first, coefficients};
+  return {out.first, torch::nullopt};
+}
+
+// Backward half: the one pass over (rows, V), with loss_grad (a one-element float
+// tensor on the device) folded in.  Logits input: `logits` is overwritten and
+// returned (cuda.cu:449); log-softmax input: a new tensor (cuda.cu:444).
+torch::Tensor apply_deferred_gradient(torch::Tensor &logits, const torch::Tensor &coefficients,
+                                      bool from_log_softmax, double grad_scale,
+                                      const torch::Tensor &loss_grad) {
+  TORCH_CHECK(logits.is_cuda() && logits.scalar_type() == torch::kFloat && logits.dim() == 2 &&
+                  logits.is_contiguous(),
+              "apply_deferred_gradient: logits must be a contiguous 2-D float32 HIP tensor");
+  const int64_t rows = logits.size(0), V = logits.size(1);
+  TORCH_CHECK(rows > 0 && V > 0 && rows <= INT32_MAX && V <= INT32_MAX,
+              "apply_deferred_gradient: bad logits shape");
+  TORCH_CHECK(coefficients.is_cuda() && coefficients.device() == logits.device() &&
+                  coefficients.scalar_type() == torch::kUInt8 && coefficients.is_contiguous() &&
+                  coefficients.numel() == (int64_t)ot_gradient_scratch_bytes(rows),
+              "apply_deferred_gradient: coefficients do not belong to these logits");
+  TORCH_CHECK(loss_grad.is_cuda() && loss_grad.device() == logits.device() &&
+                  loss_grad.scalar_type() == torch::kFloat && loss_grad.numel() == 1,
+              "apply_deferred_gradient: loss_grad must be one float32 on the device of logits");
+  c10::hip::HIPGuardMasqueradingAsCUDA device_guard(logits.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+  torch::Tensor gradient = from_log_softmax ? torch::empty_like(logits) : logits;
+  ScopedTimer timer(from_log_softmax ? "grad_logsoftmax" : "grad_logits", stream);
+  OT_CHECK(ot_gradient_apply_device_factor(logits.data_ptr<float>(), coefficients.data_ptr(), rows,
+                                           (int32_t)V, from_log_softmax, (float)grad_scale,
+                                           loss_grad.data_ptr<float>(),
+                                           gradient.data_ptr<float>(), stream));
+  return gradient;
 }
 
 // x *= loss_grad with loss_grad read on the device (no host synchronisation);
@@ -382,11 +445,21 @@ PYBIND11_MODULE(_optimized_transducer, m) {
   m.def("compute_transducer_loss", &compute_transducer_loss, py::arg("logits"),
         py::arg("targets"), py::arg("logit_lengths"), py::arg("target_lengths"),
         py::arg("blank"), py::arg("from_log_softmax"), py::arg("one_sym_per_frame"));
-  m.def("compute_transducer_loss_scaled", &compute_impl, py::arg("logits"), py::arg("targets"),
+  m.def("compute_transducer_loss_scaled", &compute_transducer_loss_scaled, py::arg("logits"), py::arg("targets"),
         py::arg("logit_lengths"), py::arg("target_lengths"), py::arg("blank"),
         py::arg("from_log_softmax"), py::arg("one_sym_per_frame"), py::arg("grad_scale"),
         "Same as compute_transducer_loss with the gradient multiplied by grad_scale in the "
         "gradient kernel (folds the `grad /= N` of reduction='mean').");
+  m.def("compute_transducer_loss_deferred", &compute_transducer_loss_deferred, py::arg("logits"),
+        py::arg("targets"), py::arg("logit_lengths"), py::arg("target_lengths"), py::arg("blank"),
+        py::arg("from_log_softmax"), py::arg("one_sym_per_frame"), py::arg("grad_scale"),
+        "Everything but the (rows, V) gradient pass: returns (scores, per-row coefficients or "
+        "None) and leaves logits untouched.");
+  m.def("apply_deferred_gradient", &apply_deferred_gradient, py::arg("logits"),
+        py::arg("coefficients"), py::arg("from_log_softmax"), py::arg("grad_scale"),
+        py::arg("loss_grad"),
+        "The (rows, V) gradient pass for the coefficients of compute_transducer_loss_deferred, "
+        "times grad_scale and the device scalar loss_grad.");
   m.def("scale_by_device_scalar_", &scale_by_device_scalar_, py::arg("x"), py::arg("factor"));
   m.def("set_profiling", &set_profiling, py::arg("on"));
   m.def("set_overlap", &set_overlap, py::arg("on"),

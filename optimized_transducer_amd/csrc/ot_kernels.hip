@@ -536,7 +536,10 @@ template <int VEC, bool FLS>
 __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
     const float *logits, float *grad, const float4 *__restrict__ coef_f,
     const int2 *__restrict__ coef_i, int64_t unit_begin, int64_t nunits, int nvec, float inv_nvec,
-    double inv_nvec_d, float scale) {
+    double inv_nvec_d, float scale, const float *__restrict__ device_factor) {
+  // optional second factor that lives on the device (the upstream gradient of the loss)
+  const float factor = device_factor ? *device_factor : 1.f;
+  if (!FLS) scale *= factor;
   // this launch covers units [unit_begin, nunits)
   const int64_t base = unit_begin + (int64_t)blockIdx.x * (kGradUnroll * kBlock);
   // base / nvec through a double reciprocal (exact below 2^53) and one correction step
@@ -580,8 +583,8 @@ __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
       if (d1 < (unsigned)VEC || d2 < (unsigned)VEC) {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-          if (d1 == (unsigned)e) y.v[e] = f.x;
-          if (d2 == (unsigned)e) y.v[e] = f.y;
+          if (d1 == (unsigned)e) y.v[e] = f.x * factor;
+          if (d2 == (unsigned)e) y.v[e] = f.y * factor;
         }
       }
     } else {
@@ -612,12 +615,24 @@ __global__ __launch_bounds__(kBlock) void scale_kernel(float *__restrict__ x, in
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
-    float4 *x4 = reinterpret_cast<float4 *>(x);
+    // spans of kScaleUnroll * 256 16-byte units: all loads of a span, then all
+    // stores, non-temporal; the tail of the last span is cut by the buffer bounds
+    constexpr int kScaleUnroll = 4;
+    constexpr int64_t kSpan = (int64_t)kScaleUnroll * kBlock;
     const int64_t n4 = n / 4;
-    for (int64_t i = tid; i < n4; i += stride) {
-      float4 v = x4[i];
-      v.x *= f; v.y *= f; v.z *= f; v.w *= f;
-      x4[i] = v;
+    for (int64_t base = (int64_t)blockIdx.x * kSpan; base < n4; base += (int64_t)gridDim.x * kSpan) {
+      const unsigned bytes = (unsigned)min(kSpan, n4 - base) * 16u;
+      const __amdgpu_buffer_rsrc_t buf = make_buffer(x + base * 4, bytes);
+      Vec<4> v[kScaleUnroll];
+#pragma unroll
+      for (int k = 0; k < kScaleUnroll; ++k)
+        v[k].load_buffer(buf, (unsigned)(k * kBlock + (int)threadIdx.x) * 16u);
+#pragma unroll
+      for (int k = 0; k < kScaleUnroll; ++k) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[k].v[e] *= f;
+        v[k].store_buffer(buf, (unsigned)(k * kBlock + (int)threadIdx.x) * 16u);
+      }
     }
     for (int64_t i = n4 * 4 + tid; i < n; i += stride) x[i] *= f;
   } else {
@@ -824,9 +839,10 @@ int ot_row_coefficients(const float *lp, const float *den, const float *alpha, c
                                    one_sym_per_frame, grad_scale, 0, rows, row_scratch, stream);
 }
 
-int ot_gradient_apply_range(const float *logits, const void *row_scratch, int64_t rows, int32_t V,
-                            int32_t from_log_softmax, float grad_scale, int64_t row_begin,
-                            int64_t row_end, float *grad, void *stream) {
+static int launch_gradient_apply(const float *logits, const void *row_scratch, int64_t rows,
+                                 int32_t V, int32_t from_log_softmax, float grad_scale,
+                                 const float *device_factor, int64_t row_begin, int64_t row_end,
+                                 float *grad, void *stream) {
   if (!row_scratch || !grad || rows <= 0 || rows > INT32_MAX || V <= 0 || row_begin < 0 ||
       row_end > rows || row_begin > row_end)
     return OT_E_BAD_ARG;
@@ -850,7 +866,7 @@ int ot_gradient_apply_range(const float *logits, const void *row_scratch, int64_
 #define OT_LAUNCH_GRAD(VEC_, FLS_)                                                            \
   hipLaunchKernelGGL((grad_flat_kernel<VEC_, FLS_>), grid, dim3(kBlock), 0, s, logits, grad,  \
                      coef_f, coef_i, unit_begin, unit_end, nvec, inv_nvec, 1.0 / (double)nvec,       \
-                     grad_scale)
+                     grad_scale, device_factor)
   if (from_log_softmax) {
     if (vec == 4) OT_LAUNCH_GRAD(4, true); else OT_LAUNCH_GRAD(1, true);
   } else {
@@ -860,10 +876,25 @@ int ot_gradient_apply_range(const float *logits, const void *row_scratch, int64_
   return launch_status();
 }
 
+int ot_gradient_apply_range(const float *logits, const void *row_scratch, int64_t rows, int32_t V,
+                            int32_t from_log_softmax, float grad_scale, int64_t row_begin,
+                            int64_t row_end, float *grad, void *stream) {
+  return launch_gradient_apply(logits, row_scratch, rows, V, from_log_softmax, grad_scale, nullptr,
+                               row_begin, row_end, grad, stream);
+}
+
 int ot_gradient_apply(const float *logits, const void *row_scratch, int64_t rows, int32_t V,
                       int32_t from_log_softmax, float grad_scale, float *grad, void *stream) {
-  return ot_gradient_apply_range(logits, row_scratch, rows, V, from_log_softmax, grad_scale, 0,
-                                 rows, grad, stream);
+  return launch_gradient_apply(logits, row_scratch, rows, V, from_log_softmax, grad_scale, nullptr,
+                               0, rows, grad, stream);
+}
+
+int ot_gradient_apply_device_factor(const float *logits, const void *row_scratch, int64_t rows,
+                                    int32_t V, int32_t from_log_softmax, float grad_scale,
+                                    const float *device_factor, float *grad, void *stream) {
+  if (!device_factor) return OT_E_BAD_ARG;
+  return launch_gradient_apply(logits, row_scratch, rows, V, from_log_softmax, grad_scale,
+                               device_factor, 0, rows, grad, stream);
 }
 
 int ot_gradient(const float *logits, const float *lp, const float *den, const float *alpha,
@@ -888,7 +919,7 @@ int ot_scale_by_device_scalar(float *x, int64_t n, const float *factor, void *st
   if (!x || !factor || n < 0) return OT_E_BAD_ARG;
   if (n == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  int64_t blocks = (n / 4 + kBlock - 1) / kBlock;
+  int64_t blocks = (n / 4 + 4 * kBlock - 1) / (4 * kBlock);
   if (blocks > 256 * 16) blocks = 256 * 16;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL(scale_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, x, n, factor);
@@ -948,7 +979,7 @@ int ot_copy_floats(const float *src, float *dst, int64_t n, void *stream) {
     return OT_E_BAD_ARG;
   if (n == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  int64_t blocks = (n / 4 + kBlock - 1) / kBlock;
+  int64_t blocks = (n / 4 + 4 * kBlock - 1) / (4 * kBlock);
   if (blocks > 256 * 16) blocks = 256 * 16;
   hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s,
                      reinterpret_cast<const float4 *>(src), reinterpret_cast<float4 *>(dst), n / 4);

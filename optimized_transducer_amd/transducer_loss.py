@@ -13,6 +13,14 @@ Differences from the reference that do not change results:
   shared tensor object forces when ``logits`` is a leaf;
 * ``TransducerLoss.__init__`` calls ``super().__init__()`` so the module can
   actually be called (the reference's class omits it, transducer_loss.py:173-188).
+
+One addition, off unless asked for: ``defer_gradient=True`` (keyword only) leaves
+``logits`` untouched in ``forward`` and makes the single pass over (rows, V) in
+``backward``, with ``loss_grad`` and ``1/N`` folded into it.  Results are the
+same; what changes is *when* ``logits`` is overwritten (in ``backward`` instead
+of ``forward``), and that a loss which is scaled or weighted before
+``backward()`` (mixed-precision loss scaling, a weighted sum of losses) costs no
+second pass over the gradient.
 """
 import torch
 
@@ -31,6 +39,7 @@ class TransducerLossFunction(torch.autograd.Function):
         from_log_softmax: bool,
         one_sym_per_frame: bool,
         reduction: str = "mean",
+        defer_gradient: bool = False,
     ) -> torch.Tensor:
         """See :func:`transducer_loss` for the arguments.
 
@@ -42,6 +51,26 @@ class TransducerLossFunction(torch.autograd.Function):
 
         batch_size = logit_lengths.size(0)
         grad_scale = 1.0 / batch_size if (reduction == "mean" and batch_size > 0) else 1.0
+
+        ctx.deferred = None
+        if defer_gradient:
+            scores, coefficients = _optimized_transducer.compute_transducer_loss_deferred(
+                logits=logits,
+                targets=targets,
+                logit_lengths=logit_lengths,
+                target_lengths=target_lengths,
+                blank=blank,
+                from_log_softmax=from_log_softmax,
+                one_sym_per_frame=one_sym_per_frame,
+                grad_scale=grad_scale,
+            )
+            if coefficients is not None:
+                # saved through autograd: an in-place change of logits before
+                # backward is then reported instead of giving a wrong gradient
+                ctx.save_for_backward(logits)
+                ctx.deferred = (coefficients, from_log_softmax, grad_scale)
+            loss = -1 * scores
+            return loss.mean() if reduction == "mean" else loss.sum()
 
         scores, grad = _optimized_transducer.compute_transducer_loss_scaled(
             logits=logits,
@@ -66,6 +95,21 @@ class TransducerLossFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, loss_grad):
         assert loss_grad.numel() == 1, loss_grad.numel()
+        no_grads = (None,) * 8  # targets ... defer_gradient
+        if ctx.deferred is not None:
+            coefficients, from_log_softmax, grad_scale = ctx.deferred
+            assert coefficients is not None, "backward through a deferred transducer loss runs once"
+            (logits,) = ctx.saved_tensors
+            ctx.deferred = (None, from_log_softmax, grad_scale)
+            factor = loss_grad.detach().to(device=logits.device, dtype=torch.float32).contiguous()
+            grad = _optimized_transducer.apply_deferred_gradient(
+                logits=logits.detach(),
+                coefficients=coefficients,
+                from_log_softmax=from_log_softmax,
+                grad_scale=grad_scale,
+                loss_grad=factor,
+            )
+            return (grad,) + no_grads
         # Hand autograd a fresh alias of the gradient buffer and drop ours: when
         # `logits` is a leaf, autograd then adopts the buffer as logits.grad
         # instead of cloning (rows, V) floats because others still hold it.
@@ -80,16 +124,7 @@ class TransducerLossFunction(torch.autograd.Function):
             _optimized_transducer.scale_by_device_scalar_(grad, loss_grad.detach().contiguous())
         else:
             grad.mul_(loss_grad)
-        return (
-            grad,  # logits
-            None,  # targets
-            None,  # logit_lengths
-            None,  # target_lengths
-            None,  # blank
-            None,  # from_log_softmax
-            None,  # one_sym_per_frame
-            None,  # reduction
-        )
+        return (grad,) + no_grads
 
 
 class TransducerLoss(torch.nn.Module):
@@ -99,10 +134,14 @@ class TransducerLoss(torch.nn.Module):
           blank: ID of the blank symbol.
           reduction: "mean" (average over the utterances of the batch) or
             "sum".  "none" is not supported (reference transducer_loss.py:133).
+
+        Set the attribute ``defer_gradient`` to True afterwards for the deferred
+        mode described in :func:`transducer_loss`.
         """
         super().__init__()
         self.blank = blank
         self.reduction = reduction
+        self.defer_gradient = False
 
     def forward(
         self,
@@ -123,6 +162,7 @@ class TransducerLoss(torch.nn.Module):
             from_log_softmax,
             one_sym_per_frame,
             self.reduction,
+            self.defer_gradient,
         )
 
 
@@ -135,6 +175,8 @@ def transducer_loss(
     from_log_softmax: bool,
     one_sym_per_frame: bool = False,
     reduction: str = "mean",
+    *,
+    defer_gradient: bool = False,
 ) -> torch.Tensor:
     """Transducer loss of a packed batch.
 
@@ -153,6 +195,11 @@ def transducer_loss(
       one_sym_per_frame: modified transducer - every arc, blank or symbol,
         advances one frame (needs U_i <= T_i - 1).
       reduction: "mean" or "sum" over the N utterances.
+      defer_gradient: not in the reference.  False: the gradient is computed
+        in the forward call, as in the reference.  True: the forward call
+        leaves ``logits`` alone and ``backward`` computes the gradient (into
+        the ``logits`` buffer for logits input), already multiplied by the
+        upstream gradient.  ``logits`` must not be modified in between.
     Returns:
       A 0-dim tensor with the reduced negative log-likelihood.
     """
@@ -165,4 +212,5 @@ def transducer_loss(
         from_log_softmax,
         one_sym_per_frame,
         reduction,
+        defer_gradient,
     )

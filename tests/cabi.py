@@ -88,13 +88,27 @@ def alpha_beta(lp, T, U, splits, max_u1, one_sym_per_frame):
 
 
 def gradient(logits, lp, den, alpha, beta, targets, T, U, splits, blank, from_log_softmax,
-             one_sym_per_frame, grad_scale=1.0, grad=None):
+             one_sym_per_frame, grad_scale=1.0, grad=None, device_factor=None):
+    """ot_gradient; with device_factor (a one-element device tensor) the two launches
+    ot_row_coefficients + ot_gradient_apply_device_factor instead."""
     rows, V = logits.shape
     if grad is None:
         grad = torch.full((rows, V), float("nan"), dtype=torch.float32, device=logits.device)
     cols = targets.shape[1]
     scratch = torch.empty(lib().ot_gradient_scratch_bytes(ctypes.c_int64(rows)), dtype=torch.uint8,
                           device=logits.device)
+    if device_factor is not None:
+        check(lib().ot_row_coefficients(
+            ptr(lp), ptr(den), ptr(alpha), ptr(beta), ptr(targets if cols else None), ptr(T), ptr(U),
+            ptr(splits), ctypes.c_int32(T.numel()), ctypes.c_int32(cols), ctypes.c_int64(rows),
+            ctypes.c_int32(blank), ctypes.c_int32(int(from_log_softmax)),
+            ctypes.c_int32(int(one_sym_per_frame)), ctypes.c_float(grad_scale), ptr(scratch),
+            stream()))
+        check(lib().ot_gradient_apply_device_factor(
+            ptr(logits), ptr(scratch), ctypes.c_int64(rows), ctypes.c_int32(V),
+            ctypes.c_int32(int(from_log_softmax)), ctypes.c_float(grad_scale), ptr(device_factor),
+            ptr(grad), stream()))
+        return grad
     check(lib().ot_gradient(ptr(logits), ptr(lp), ptr(den), ptr(alpha), ptr(beta),
                             ptr(targets if cols else None), ptr(T), ptr(U), ptr(splits),
                             ctypes.c_int32(T.numel()), ctypes.c_int32(cols), ctypes.c_int64(rows),

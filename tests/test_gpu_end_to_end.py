@@ -217,6 +217,116 @@ def test_two_stream_schedule_gives_the_same_bits(device):
         assert torch.equal(loss, out[0][0]) and torch.equal(grad, out[0][1])
 
 
+@pytest.mark.parametrize("fls,osf", MODES)
+def test_deferred_gradient_mode(fls, osf, device):
+    # defer_gradient=True: forward leaves logits alone, backward makes the one (rows, V)
+    # pass with loss_grad folded in; same numbers as the reference order of operations
+    import optimized_transducer_amd as ot
+    w = workloads.tiny(from_log_softmax=fls, one_sym_per_frame=osf)
+    x = w.logits_numpy()
+    tg, T, U = _dev(w.targets, device), _dev(w.logit_lengths, device), _dev(w.target_lengths, device)
+
+    def run(defer, upstream, reduction="mean", module=False):
+        logits = _dev(x, device).requires_grad_(True)
+        if module:
+            m = ot.TransducerLoss(blank=w.blank, reduction=reduction)
+            m.defer_gradient = defer
+            loss = m(logits, tg, T, U, fls, osf)
+        else:
+            loss = ot.transducer_loss(logits, tg, T, U, w.blank, fls, one_sym_per_frame=osf,
+                                      reduction=reduction, defer_gradient=defer)
+        untouched = np.array_equal(logits.detach().cpu().numpy(), x)
+        (loss * upstream).backward()
+        return loss.detach(), logits, untouched
+
+    for upstream, reduction in ((1.0, "mean"), (0.5, "sum"), (3.0, "mean")):
+        l0, a, _ = run(False, upstream, reduction)
+        l1, b, untouched = run(True, upstream, reduction)
+        assert untouched  # forward wrote nothing
+        assert torch.equal(l0, l1)
+        if upstream in (1.0, 0.5):  # power-of-two factors: the two orders round alike
+            assert torch.equal(a.grad, b.grad)
+        assert torch.allclose(a.grad, b.grad, rtol=1e-6, atol=1e-30)
+        if fls:
+            assert np.array_equal(b.detach().cpu().numpy(), x)  # log-softmax input survives
+            assert b.grad.data_ptr() != b.data_ptr()
+        else:
+            assert b.grad.data_ptr() == b.data_ptr()  # written in place, adopted by autograd
+    l2, c, _ = run(True, 3.0, module=True)
+    assert torch.equal(l2, l1) and torch.equal(c.grad, b.grad)
+    want_loss, want = oracle.transducer_loss(x.copy(), w.targets, w.logit_lengths, w.target_lengths,
+                                             w.blank, fls, osf, "mean", loss_grad=3.0)
+    assert np.allclose(l2.item(), want_loss, rtol=RTOL, atol=ATOL)
+    s, _ = oracle.compute_transducer_loss(x.copy(), w.targets, w.logit_lengths, w.target_lengths,
+                                          w.blank, fls, osf)
+    scale = 3.0 / w.N
+    tol = scale * helpers.lattice_noise_tolerance(want / scale,
+                                                  helpers.per_row(s, w.logit_lengths, w.target_lengths))
+    assert (np.abs(c.grad.cpu().numpy() - want) <= tol).all()
+
+    # no gradient wanted: nothing kept, nothing written
+    plain = _dev(x, device)
+    l3 = ot.transducer_loss(plain, tg, T, U, w.blank, fls, one_sym_per_frame=osf,
+                            defer_gradient=True)
+    assert not l3.requires_grad and torch.equal(l3, l1)
+    # logits changed between forward and backward: autograd reports it
+    logits = _dev(x, device).requires_grad_(True)
+    h = logits * 1.0
+    loss = ot.transducer_loss(h, tg, T, U, w.blank, fls, one_sym_per_frame=osf, defer_gradient=True)
+    h.add_(1.0)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        loss.backward()
+
+
+def test_side_stream_and_unaligned_views(device):
+    # the launches follow torch's current stream (cuda.cu:92), and a contiguous view
+    # that starts 4 bytes into an allocation (16-byte vector accesses impossible)
+    # gives the same result as an aligned tensor
+    import optimized_transducer_amd as ot
+    rng = np.random.default_rng(77)
+    T, U, tg, x = helpers.random_batch(rng, 5, 30, 12, 40)
+    tg = np.where(tg == 0, 1, tg).astype(np.int32)
+    dtg, dT, dU = _dev(tg, device), _dev(T, device), _dev(U, device)
+    want_loss, want = oracle.transducer_loss(x.copy(), tg, T, U, 0, False, False, "sum")
+
+    def check(loss, grad):
+        assert np.allclose(loss.item(), want_loss, rtol=RTOL, atol=ATOL)
+        s, _ = oracle.compute_transducer_loss(x.copy(), tg, T, U, 0, False, False)
+        tol = helpers.lattice_noise_tolerance(want, helpers.per_row(s, T, U))
+        assert (np.abs(grad.cpu().numpy() - want) <= tol).all()
+
+    side = torch.cuda.Stream(device=device)
+    logits = _dev(x, device).requires_grad_(True)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        loss = ot.transducer_loss(logits, dtg, dT, dU, 0, False, reduction="sum")
+        loss.backward()
+    side.synchronize()
+    check(loss, logits.grad)
+    ref_grad = logits.grad.clone()
+
+    flat = torch.zeros(x.size + 1, device=device)
+    view = flat[1:].view(x.shape)
+    view.copy_(_dev(x, device))
+    assert view.data_ptr() % 16 == 4 and view.is_contiguous()
+    view.requires_grad_(True)
+    loss = ot.transducer_loss(view, dtg, dT, dU, 0, False, reduction="sum")
+    loss.backward()
+    check(loss, view.grad)
+    assert torch.allclose(view.grad, ref_grad, rtol=1e-4, atol=1e-6)  # scalar vs vector code path
+    assert flat[0].item() == 0  # nothing written in front of the view
+
+    # log-softmax input on the view: gradient is a fresh (aligned) tensor
+    xl = helpers.log_softmax32(x)
+    view2 = torch.zeros(x.size + 1, device=device)[1:].view(x.shape)
+    view2.copy_(_dev(xl, device))
+    view2.requires_grad_(True)
+    a = _dev(xl, device).requires_grad_(True)
+    ot.transducer_loss(view2, dtg, dT, dU, 0, True, reduction="sum").backward()
+    ot.transducer_loss(a, dtg, dT, dU, 0, True, reduction="sum").backward()
+    assert torch.equal(view2.grad, a.grad)
+
+
 # ------------------------------------------------------------------ full sizes
 FULL = [
     ("asr", lambda: workloads.asr_batch()),

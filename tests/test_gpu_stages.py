@@ -138,6 +138,11 @@ def test_gradient_kernels_given_oracle_lattice(case, fls, device):
     # folded scale (reduction="mean"): multiplication by 1/N, exact for a power of two
     got4 = cabi.gradient(*args, grad_scale=0.25).cpu().numpy()
     assert (got4 == got * np.float32(0.25)).all()
+    # one more factor, read from device memory by the kernel (the upstream gradient of the
+    # loss in the deferred mode); powers of two keep the comparison exact
+    four = torch.full((1,), 4.0, device=device)
+    got2 = cabi.gradient(*args, grad_scale=2.0, device_factor=four).cpu().numpy()
+    assert (got2 == got * np.float32(8.0)).all()
     if not fls:
         # in place: the logits buffer itself receives the gradient (cuda.cu:449)
         buf = dx.clone()

@@ -64,8 +64,12 @@ def test_python_entry_points_keep_the_reference_signatures():
     import optimized_transducer_amd as ot
     # optimized_transducer/python/optimized_transducer/transducer_loss.py:312-321
     sig = inspect.signature(ot.transducer_loss)
-    assert list(sig.parameters) == ["logits", "targets", "logit_lengths", "target_lengths", "blank",
-                                    "from_log_softmax", "one_sym_per_frame", "reduction"]
+    ref_names = ["logits", "targets", "logit_lengths", "target_lengths", "blank",
+                 "from_log_softmax", "one_sym_per_frame", "reduction"]
+    assert list(sig.parameters)[:8] == ref_names
+    for extra in list(sig.parameters)[8:]:  # additions: keyword only, off by default
+        assert sig.parameters[extra].kind is inspect.Parameter.KEYWORD_ONLY
+        assert sig.parameters[extra].default is False
     assert sig.parameters["one_sym_per_frame"].default is False
     assert sig.parameters["reduction"].default == "mean"
     assert sig.parameters["from_log_softmax"].default is inspect.Parameter.empty
