@@ -219,6 +219,55 @@ int ot_transducer_loss(const float *logits, const int32_t *targets,
                        size_t workspace_bytes, float *scores, float *grad,
                        ot_batch_status *status, void *stream);
 
+/* ---- packed joiner input: the data format on the input side of the loss ----
+ *
+ * The loss consumes the joiner output for the valid (t, u) cells only, in the
+ * packed row order above.  The reference leaves producing the joiner INPUT in
+ * that order to its caller and shows it with Python lists and torch.cat
+ * (README.md:166-177):
+ *   x = cat_b (enc[b, :T_b, None, :] + dec[b, None, :U_b+1, :]).reshape(-1, D)
+ *   activation = tanh(x)
+ * The functions below do that, and its gradient, from the padded tensors
+ *   enc (N, t_stride, D), t_stride >= max_b T_b        (encoder output)
+ *   dec (N, u_stride, D), u_stride >= max_b U_b + 1    (prediction network output)
+ * all float32 and contiguous. */
+#define OT_ACT_NONE 0 /* out = enc + dec                                      */
+#define OT_ACT_TANH 1 /* out = tanh(enc + dec)                                */
+#define OT_JOINER_TILE_FRAMES 16 /* frames per partial decoder sum            */
+
+/* row_index: (rows, 2) int32, 8-byte aligned: for packed row r of utterance b,
+ * cell (t, u): {b*t_stride + t, b*u_stride + u}, the source rows in enc and
+ * dec viewed as (N*t_stride, D) and (N*u_stride, D); {-1, -1} for rows beyond
+ * row_splits[N].  Depends on the lengths only: compute once per batch. */
+int ot_joiner_rows(const int32_t *logit_lengths, const int32_t *target_lengths,
+                   const int32_t *row_splits, int32_t N, int64_t rows,
+                   int32_t t_stride, int32_t u_stride, int32_t *row_index,
+                   void *stream);
+
+/* out (rows, D): out[r] = act(enc[row_index[r][0]] + dec[row_index[r][1]]);
+ * one streaming pass, 4*D bytes written per row. */
+int ot_joiner_pack(const float *enc, const float *dec, const int32_t *row_index,
+                   int64_t rows, int32_t D, int32_t activation, float *out,
+                   void *stream);
+
+/* Gradient of ot_joiner_pack: given grad_out (rows, D) = d loss / d out,
+ *   grad_enc[b,t,:] = sum_u grad_out[row(b,t,u)] * act'(enc[b,t] + dec[b,u])
+ *   grad_dec[b,u,:] = sum_t (the same terms)
+ * and zeros in the padding (t >= T_b, u > U_b); both outputs are written in
+ * full.  One pass over grad_out; the decoder sums go through per-16-frame
+ * partial sums in `workspace` (16-byte aligned, ot_joiner_unpack_workspace_bytes)
+ * and are added in a fixed order, so results do not vary from run to run.
+ * enc and dec are read only for OT_ACT_TANH (may be NULL otherwise). */
+size_t ot_joiner_unpack_workspace_bytes(int32_t N, int32_t t_stride,
+                                        int32_t u_stride, int32_t D);
+int ot_joiner_unpack_grad(const float *grad_out, const float *enc,
+                          const float *dec, const int32_t *logit_lengths,
+                          const int32_t *target_lengths,
+                          const int32_t *row_splits, int32_t N, int32_t t_stride,
+                          int32_t u_stride, int32_t D, int32_t activation,
+                          void *workspace, size_t workspace_bytes,
+                          float *grad_enc, float *grad_dec, void *stream);
+
 /* Plain device-to-device copy kernel of n floats; used to calibrate profiler
  * byte counters against a transfer of known size. */
 int ot_copy_floats(const float *src, float *dst, int64_t n, void *stream);

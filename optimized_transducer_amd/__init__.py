@@ -16,5 +16,7 @@ except ImportError as e:  # pragma: no cover - exercised only on an unbuilt tree
     ) from e
 
 from .transducer_loss import TransducerLoss, TransducerLossFunction, transducer_loss  # noqa: E402,F401
+from .joiner import PackJoinerFunction, pack_joiner  # noqa: E402,F401
 
-__all__ = ["TransducerLoss", "TransducerLossFunction", "transducer_loss"]
+__all__ = ["TransducerLoss", "TransducerLossFunction", "transducer_loss", "PackJoinerFunction",
+           "pack_joiner"]

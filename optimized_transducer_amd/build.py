@@ -34,9 +34,9 @@ def _run(cmd):
 
 
 def build_kernels():
-    src = os.path.join(CSRC, "ot_kernels.hip")
+    srcs = [os.path.join(CSRC, f) for f in ("ot_kernels.hip", "ot_joiner.hip")]
     _run([os.path.join(ROCM, "bin", "hipcc")] + HIPCC_FLAGS +
-         ["-I", INCLUDE, "-I", CSRC, src, "-o", KERNEL_LIB])
+         ["-I", INCLUDE, "-I", CSRC] + srcs + ["-o", KERNEL_LIB])
     return KERNEL_LIB
 
 

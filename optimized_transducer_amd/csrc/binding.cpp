@@ -438,6 +438,133 @@ void scale_by_device_scalar_(torch::Tensor &x, const torch::Tensor &factor) {
                                      stream));
 }
 
+// ---- packed joiner input (the reference's README.md:166-177, done on the device) ----
+
+int activation_code(const std::string &name) {
+  if (name == "none") return OT_ACT_NONE;
+  if (name == "tanh") return OT_ACT_TANH;
+  TORCH_CHECK(false, "activation must be 'none' or 'tanh', got '", name, "'");
+  return -1;
+}
+
+void check_joiner_inputs(const torch::Tensor &enc, const torch::Tensor &dec,
+                         const torch::Tensor &logit_lengths, const torch::Tensor &target_lengths) {
+  TORCH_CHECK(enc.is_cuda() && dec.is_cuda() && logit_lengths.is_cuda() && target_lengths.is_cuda() &&
+                  enc.device() == dec.device() && enc.device() == logit_lengths.device() &&
+                  enc.device() == target_lengths.device(),
+              "pack_joiner: all tensors must be on the same HIP device (this build has no CPU "
+              "implementation)");
+  TORCH_CHECK(enc.scalar_type() == torch::kFloat && dec.scalar_type() == torch::kFloat,
+              "pack_joiner: encoder_out and decoder_out must be float32");
+  TORCH_CHECK(logit_lengths.scalar_type() == torch::kInt32 &&
+                  target_lengths.scalar_type() == torch::kInt32,
+              "pack_joiner: logit_lengths and target_lengths must be int32");
+  TORCH_CHECK(enc.dim() == 3 && dec.dim() == 3 && logit_lengths.dim() == 1 &&
+                  target_lengths.dim() == 1,
+              "pack_joiner: expected encoder_out (N, T, D), decoder_out (N, U+1, D) and 1-D lengths");
+  TORCH_CHECK(enc.is_contiguous() && dec.is_contiguous() && logit_lengths.is_contiguous() &&
+                  target_lengths.is_contiguous(),
+              "pack_joiner: tensors must be contiguous");
+  const int64_t N = enc.size(0);
+  TORCH_CHECK(N > 0 && dec.size(0) == N && logit_lengths.size(0) == N && target_lengths.size(0) == N,
+              "pack_joiner: batch sizes differ: ", enc.size(0), ", ", dec.size(0), ", ",
+              logit_lengths.size(0), ", ", target_lengths.size(0));
+  TORCH_CHECK(enc.size(2) == dec.size(2) && enc.size(2) > 0,
+              "pack_joiner: encoder_out and decoder_out differ in the last dimension: ", enc.size(2),
+              " vs ", dec.size(2));
+  TORCH_CHECK(enc.size(1) > 0 && dec.size(1) > 0 && N * enc.size(1) <= INT32_MAX &&
+                  N * dec.size(1) <= INT32_MAX && enc.size(2) <= INT32_MAX && N <= 65535,
+              "pack_joiner: tensor sizes out of range");
+}
+
+// (packed (rows, D), row_splits (N+1) int32, row_index (rows, 2) int32)
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> joiner_pack(
+    const torch::Tensor &enc, const torch::Tensor &dec, const torch::Tensor &logit_lengths,
+    const torch::Tensor &target_lengths, const std::string &activation) {
+  const int act = activation_code(activation);
+  check_joiner_inputs(enc, dec, logit_lengths, target_lengths);
+  const int64_t N = enc.size(0), Tmax = enc.size(1), U1max = dec.size(1), D = enc.size(2);
+  c10::hip::HIPGuardMasqueradingAsCUDA device_guard(enc.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+
+  torch::Tensor row_splits = torch::empty({N + 1}, logit_lengths.options());
+  torch::Tensor status_host = torch::empty(
+      {(int64_t)sizeof(ot_batch_status)},
+      torch::TensorOptions().dtype(torch::kUInt8).device(torch::kCPU).pinned_memory(true));
+  void *status_dev = nullptr;
+  OT_CHECK_HIP(hipHostGetDevicePointer(&status_dev, status_host.data_ptr(), 0));
+  {
+    ScopedTimer timer("prepare", stream);
+    OT_CHECK(ot_row_splits(logit_lengths.data_ptr<int32_t>(), target_lengths.data_ptr<int32_t>(),
+                           nullptr, (int32_t)N, 0, row_splits.data_ptr<int32_t>(), nullptr,
+                           static_cast<ot_batch_status *>(status_dev), stream));
+  }
+  EventGuard ready;
+  OT_CHECK_HIP(hipEventRecord(ready.ev, stream));
+  OT_CHECK_HIP(hipEventSynchronize(ready.ev));  // the output's size is a batch fact
+  const ot_batch_status st = *reinterpret_cast<const ot_batch_status *>(status_host.data_ptr());
+  TORCH_CHECK(st.logit_len_min >= 1 && st.target_len_min >= 0,
+              "pack_joiner: expect logit_lengths >= 1 and target_lengths >= 0, but the minima are ",
+              st.logit_len_min, " and ", st.target_len_min);
+  TORCH_CHECK(st.logit_len_max <= Tmax, "pack_joiner: logit_lengths.max() is ", st.logit_len_max,
+              " but encoder_out has ", Tmax, " frames");
+  TORCH_CHECK((int64_t)st.target_len_max + 1 <= U1max, "pack_joiner: target_lengths.max() + 1 is ",
+              (int64_t)st.target_len_max + 1, " but decoder_out has ", U1max, " positions");
+  const int64_t rows = st.sum_tu;
+  TORCH_CHECK(rows > 0 && rows <= INT32_MAX, "pack_joiner: sum of T * (U + 1) is ", rows,
+              ", outside (0, 2^31)");
+
+  torch::Tensor row_index = torch::empty({rows, 2}, logit_lengths.options());
+  torch::Tensor out = torch::empty({rows, D}, enc.options());
+  {
+    ScopedTimer timer("joiner_rows", stream);
+    OT_CHECK(ot_joiner_rows(logit_lengths.data_ptr<int32_t>(), target_lengths.data_ptr<int32_t>(),
+                            row_splits.data_ptr<int32_t>(), (int32_t)N, rows, (int32_t)Tmax,
+                            (int32_t)U1max, row_index.data_ptr<int32_t>(), stream));
+  }
+  {
+    ScopedTimer timer("joiner_pack", stream);
+    OT_CHECK(ot_joiner_pack(enc.data_ptr<float>(), dec.data_ptr<float>(),
+                            row_index.data_ptr<int32_t>(), rows, (int32_t)D, act,
+                            out.data_ptr<float>(), stream));
+  }
+  return {out, row_splits, row_index};
+}
+
+// (grad_encoder_out (N, T, D), grad_decoder_out (N, U+1, D)) for grad_out (rows, D)
+std::pair<torch::Tensor, torch::Tensor> joiner_unpack_grad(
+    const torch::Tensor &grad_out, const torch::Tensor &enc, const torch::Tensor &dec,
+    const torch::Tensor &logit_lengths, const torch::Tensor &target_lengths,
+    const torch::Tensor &row_splits, const std::string &activation) {
+  const int act = activation_code(activation);
+  check_joiner_inputs(enc, dec, logit_lengths, target_lengths);
+  const int64_t N = enc.size(0), Tmax = enc.size(1), U1max = dec.size(1), D = enc.size(2);
+  TORCH_CHECK(grad_out.is_cuda() && grad_out.device() == enc.device() &&
+                  grad_out.scalar_type() == torch::kFloat && grad_out.dim() == 2 &&
+                  grad_out.size(1) == D && grad_out.is_contiguous(),
+              "pack_joiner backward: the gradient must be a contiguous float32 (rows, ", D,
+              ") tensor on the device of encoder_out");
+  TORCH_CHECK(row_splits.is_cuda() && row_splits.device() == enc.device() &&
+                  row_splits.scalar_type() == torch::kInt32 && row_splits.dim() == 1 &&
+                  row_splits.size(0) == N + 1 && row_splits.is_contiguous(),
+              "pack_joiner backward: row_splits must be the (N+1,) int32 tensor of the forward call");
+  c10::hip::HIPGuardMasqueradingAsCUDA device_guard(enc.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+  const size_t ws_bytes =
+      ot_joiner_unpack_workspace_bytes((int32_t)N, (int32_t)Tmax, (int32_t)U1max, (int32_t)D);
+  torch::Tensor workspace = torch::empty({(int64_t)ws_bytes}, enc.options().dtype(torch::kUInt8));
+  torch::Tensor grad_enc = torch::empty_like(enc);
+  torch::Tensor grad_dec = torch::empty_like(dec);
+  ScopedTimer timer("joiner_unpack_grad", stream);
+  OT_CHECK(ot_joiner_unpack_grad(grad_out.data_ptr<float>(), enc.data_ptr<float>(),
+                                 dec.data_ptr<float>(), logit_lengths.data_ptr<int32_t>(),
+                                 target_lengths.data_ptr<int32_t>(), row_splits.data_ptr<int32_t>(),
+                                 (int32_t)N, (int32_t)Tmax, (int32_t)U1max, (int32_t)D, act,
+                                 workspace.data_ptr(), ws_bytes, grad_enc.data_ptr<float>(),
+                                 grad_dec.data_ptr<float>(), stream));
+  return {grad_enc, grad_dec};
+}
+
 }  // namespace
 
 PYBIND11_MODULE(_optimized_transducer, m) {
@@ -461,6 +588,14 @@ PYBIND11_MODULE(_optimized_transducer, m) {
         "The (rows, V) gradient pass for the coefficients of compute_transducer_loss_deferred, "
         "times grad_scale and the device scalar loss_grad.");
   m.def("scale_by_device_scalar_", &scale_by_device_scalar_, py::arg("x"), py::arg("factor"));
+  m.def("joiner_pack", &joiner_pack, py::arg("encoder_out"), py::arg("decoder_out"),
+        py::arg("logit_lengths"), py::arg("target_lengths"), py::arg("activation"),
+        "Packed joiner input act(enc[b,t] + dec[b,u]) for the valid (t, u) cells, in the row order "
+        "of the loss; returns (packed (rows, D), row_splits, row_index).");
+  m.def("joiner_unpack_grad", &joiner_unpack_grad, py::arg("grad_out"), py::arg("encoder_out"),
+        py::arg("decoder_out"), py::arg("logit_lengths"), py::arg("target_lengths"),
+        py::arg("row_splits"), py::arg("activation"),
+        "Gradient of joiner_pack: (grad_encoder_out, grad_decoder_out).");
   m.def("set_profiling", &set_profiling, py::arg("on"));
   m.def("set_overlap", &set_overlap, py::arg("on"),
         "Run the lattice kernel of one half of a large batch on a second stream while the "

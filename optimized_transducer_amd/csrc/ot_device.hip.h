@@ -217,6 +217,11 @@ template <> struct Vec<4> {
     const f32x4 x = {v[0], v[1], v[2], v[3]};
     *reinterpret_cast<f32x4 *>(p) = x;
   }
+  // ordinary load, for data that is re-read from cache
+  __device__ __forceinline__ void load_cached(const float *p) {
+    const f32x4 x = *reinterpret_cast<const f32x4 *>(p);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  }
   __device__ __forceinline__ void load_lds(const float *p) {
     const f32x4 x = *reinterpret_cast<const f32x4 *>(p);
     v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
@@ -244,6 +249,7 @@ template <> struct Vec<1> {
   __device__ __forceinline__ void store(float *p) const { *p = v[0]; }
   __device__ __forceinline__ void store_stream(float *p) const { __builtin_nontemporal_store(v[0], p); }
   __device__ __forceinline__ void load_lds(const float *p) { v[0] = *p; }
+  __device__ __forceinline__ void load_cached(const float *p) { v[0] = *p; }
   __device__ __forceinline__ void load_buffer(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
     v[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, kAuxStream));
   }

@@ -1,0 +1,388 @@
+// Packed joiner input for the transducer loss, and its gradient (gfx950).
+//
+// The loss takes the joiner output for the valid (t, u) cells only, utterances
+// concatenated: row_splits[b] + t*(U_b+1) + u.  The reference leaves building
+// the joiner's *input* in that layout to the caller and shows it with Python
+// lists (README.md:166-177):
+//     x = cat([ (enc[b,:T_b].unsqueeze(1) + dec[b,:U_b+1].unsqueeze(0)).reshape(-1, D) ])
+//     activation = tanh(x)
+// The kernels here do the same from the padded encoder / decoder outputs in one
+// pass each way:
+//   joiner_rows_kernel         row -> (encoder frame, decoder position), 8 B/row
+//   joiner_pack_kernel         out[row] = act(enc[b,t] + dec[b,u]); write-bound
+//   joiner_unpack_grad_kernel  one pass over d(out): complete sums over u for
+//                              the encoder, sums over 16 frames for the decoder
+//   joiner_dec_reduce_kernel   adds the per-16-frame partial sums, fixed order
+// Sums are taken in a fixed order, so results are the same bits on every run.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ot_device.hip.h"
+#include "ot_transducer.h"
+
+namespace ot {
+
+// tanh with a relative error of a few ulp over the whole range: the odd series
+// below |x| = 0.25 (where 1 - e^-2|x| cancels), the exponential form elsewhere.
+__device__ __forceinline__ float tanh_dev(float x) {
+  const float ax = __builtin_fabsf(x);
+  const float x2 = x * x;
+  // x - x^3/3 + 2x^5/15 - 17x^7/315 + 62x^9/2835; next term 1382x^11/155925 < 1e-8 * x at 0.25
+  const float small =
+      x * (1.f + x2 * (-0.333333343f +
+                       x2 * (0.13333334f + x2 * (-0.053968254f + x2 * 0.021869488f))));
+  const float e = __builtin_amdgcn_exp2f(ax * -2.88539004325866699219f);  // exp(-2|x|)
+  const float big = __builtin_copysignf((1.f - e) * __builtin_amdgcn_rcpf(1.f + e), x);
+  return ax < 0.25f ? small : big;
+}
+
+template <int ACT>
+__device__ __forceinline__ float activate(float s) {
+  return ACT == OT_ACT_TANH ? tanh_dev(s) : s;
+}
+// d act(s) / d s
+template <int ACT>
+__device__ __forceinline__ float activate_slope(float s) {
+  if (ACT == OT_ACT_TANH) {
+    const float a = tanh_dev(s);
+    return 1.f - a * a;
+  }
+  return 1.f;
+}
+
+// ---------------------------------------------------------------------------
+// row -> source rows of the padded encoder / decoder outputs
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void joiner_rows_kernel(
+    const int32_t *__restrict__ logit_lengths, const int32_t *__restrict__ target_lengths,
+    const int32_t *__restrict__ row_splits, int N, int64_t rows, int t_stride, int u_stride,
+    int2 *__restrict__ row_index) {
+  __shared__ BlockUtterances bu;
+  const int64_t row_first = (int64_t)blockIdx.x * kBlock;
+  const int64_t row_end = min(rows, row_first + kBlock);
+  bu.load(row_splits, N, row_first, row_end - 1);
+  const int64_t row = row_first + threadIdx.x;
+  if (row >= row_end) return;
+  int2 idx = make_int2(-1, -1);  // rows beyond the batch (inconsistent sizes): no source
+  if (row < (int64_t)row_splits[N]) {
+    const Cell c = decode_row(bu, row, logit_lengths, target_lengths);
+    if (c.t < t_stride && c.u < u_stride) idx = make_int2(c.b * t_stride + c.t, c.b * u_stride + c.u);
+  }
+  row_index[row] = idx;
+}
+
+// ---------------------------------------------------------------------------
+// forward: flat pass over the (rows, D) output in units of VEC floats
+// ---------------------------------------------------------------------------
+constexpr int kPackUnroll = 2;
+
+template <int VEC, int ACT>
+__global__ __launch_bounds__(kBlock) void joiner_pack_kernel(
+    const float *__restrict__ enc, const float *__restrict__ dec,
+    const int2 *__restrict__ row_index, float *__restrict__ out, int64_t nunits, int nvec,
+    float inv_nvec, double inv_nvec_d) {
+  const int64_t base = (int64_t)blockIdx.x * (kPackUnroll * kBlock);
+  // base / nvec through a double reciprocal (exact below 2^53) and one correction step
+  int64_t row_base = (int64_t)((double)base * inv_nvec_d);
+  {
+    const int64_t r = base - row_base * nvec;
+    if (r < 0) --row_base; else if (r >= nvec) ++row_base;
+  }
+  const int rem_base = (int)(base - row_base * nvec);
+  const unsigned span_bytes =
+      (unsigned)min((int64_t)(kPackUnroll * kBlock), nunits - base) * (VEC * 4u);
+  const __amdgpu_buffer_rsrc_t out_buf = make_buffer(out + base * VEC, span_bytes);
+  const int64_t last_row = (nunits - 1) / nvec;
+#pragma unroll
+  for (int k = 0; k < kPackUnroll; ++k) {
+    const int local = k * kBlock + (int)threadIdx.x;
+    const int idx = rem_base + local;  // < nvec + kPackUnroll*256: exact in float
+    int q = (int)((float)idx * inv_nvec);
+    if (q * nvec > idx) --q; else if ((q + 1) * nvec <= idx) ++q;
+    const int col = (idx - q * nvec) * VEC;
+    const int64_t row = min(row_base + q, last_row);
+    const int2 src = row_index[row];
+    Vec<VEC> y;
+    if (src.x >= 0) {
+      Vec<VEC> e, d;
+      e.load_cached(enc + ((int64_t)src.x * nvec * VEC + col));
+      d.load_cached(dec + ((int64_t)src.y * nvec * VEC + col));
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) y.v[i] = activate<ACT>(e.v[i] + d.v[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) y.v[i] = 0.f;
+    }
+    y.store_buffer(out_buf, (unsigned)local * (VEC * 4u));
+  }
+}
+
+// ---------------------------------------------------------------------------
+// backward
+// ---------------------------------------------------------------------------
+constexpr int kTileFrames = OT_JOINER_TILE_FRAMES;  // frames per workgroup
+constexpr int kSlabLanes = 16;                      // lanes across the columns of a slab
+constexpr int kUPhases = kBlock / kSlabLanes;       // positions u in flight per workgroup
+
+// One workgroup: utterance b = blockIdx.z, frames [t0, t0 + 16), columns
+// [slab*16*VEC, (slab+1)*16*VEC).  Thread (phase, lane): columns lane*VEC.., and
+// the positions u = phase, phase + 16, ...  For one u it loads the 16 frames'
+// values (16 independent loads), adds them up for the decoder and into 16
+// per-frame accumulators for the encoder.  The encoder sums of the workgroup's
+// threads are then added through DPP/LDS in a fixed order.
+template <int VEC, int ACT>
+__global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
+    const float *__restrict__ grad_out, const float *__restrict__ enc,
+    const float *__restrict__ dec, const int32_t *__restrict__ logit_lengths,
+    const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
+    int t_stride, int u_stride, int D, float *__restrict__ grad_enc,
+    float *__restrict__ dec_partial) {
+  __shared__ __attribute__((aligned(16))) float s_enc[kTileFrames][kSlabLanes * VEC];
+  __shared__ __attribute__((aligned(16))) float s_red[kWavesPerBlock][kTileFrames][kSlabLanes * VEC];
+  const int b = blockIdx.z;
+  const int t0 = blockIdx.y * kTileFrames;
+  const int lane = threadIdx.x & (kSlabLanes - 1);
+  const int phase = threadIdx.x / kSlabLanes;
+  const int col = (blockIdx.x * kSlabLanes + lane) * VEC;
+  const bool col_ok = col < D;  // D is a multiple of VEC
+  const int T = min(logit_lengths[b], t_stride);
+  const int U1 = min(target_lengths[b] + 1, u_stride);
+  const int64_t row0 = row_splits[b];
+  const int ntiles = gridDim.y;
+
+  // frames of this tile that exist; the rest of the tile (padding of the encoder
+  // output) gets zeros
+  const int nframes = max(0, min(kTileFrames, T - t0));
+  if (ACT != OT_ACT_NONE) {
+    for (int i = phase; i < kTileFrames; i += kUPhases) {
+      Vec<VEC> e;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) e.v[k] = 0.f;
+      if (i < nframes && col_ok) e.load_cached(enc + ((int64_t)(b * t_stride + t0 + i) * D + col));
+      e.store_lds(&s_enc[i][lane * VEC]);
+    }
+    __syncthreads();
+  }
+
+  Vec<VEC> acc[kTileFrames];
+#pragma unroll
+  for (int i = 0; i < kTileFrames; ++i)
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc[i].v[k] = 0.f;
+
+  if (nframes > 0 && col_ok) {
+    const int64_t frame_stride = (int64_t)U1 * D;
+    for (int u = phase; u < U1; u += kUPhases) {
+      const float *p = grad_out + ((row0 + (int64_t)t0 * U1 + u) * D + col);
+      Vec<VEC> g[kTileFrames];
+#pragma unroll
+      for (int i = 0; i < kTileFrames; ++i) {
+        if (i < nframes) {
+          g[i].load(p + i * frame_stride);
+        } else {
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) g[i].v[k] = 0.f;
+        }
+      }
+      Vec<VEC> d, sum;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) sum.v[k] = 0.f;
+      if (ACT != OT_ACT_NONE) d.load_cached(dec + ((int64_t)(b * u_stride + u) * D + col));
+#pragma unroll
+      for (int i = 0; i < kTileFrames; ++i) {
+        if (ACT != OT_ACT_NONE) {
+          Vec<VEC> e;
+          e.load_lds(&s_enc[i][lane * VEC]);
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) g[i].v[k] *= activate_slope<ACT>(e.v[k] + d.v[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+          sum.v[k] += g[i].v[k];
+          acc[i].v[k] += g[i].v[k];
+        }
+      }
+      sum.store(dec_partial + ((((int64_t)b * ntiles + blockIdx.y) * u_stride + u) * D + col));
+    }
+  }
+
+  // encoder: add the 4 phases of a wave (lanes l, l+16, l+32, l+48), then the waves
+#pragma unroll
+  for (int i = 0; i < kTileFrames; ++i)
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      float v = acc[i].v[k];
+      v += __shfl_xor(v, 16, kWave);
+      v += __shfl_xor(v, 32, kWave);
+      acc[i].v[k] = v;
+    }
+  const int wave = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) < kSlabLanes) {
+#pragma unroll
+    for (int i = 0; i < kTileFrames; ++i) acc[i].store_lds(&s_red[wave][i][lane * VEC]);
+  }
+  __syncthreads();
+  // 16 frames x 16 lanes = 256 (frame, lane) pairs: one per thread
+  {
+    const int i = threadIdx.x / kSlabLanes, l = threadIdx.x & (kSlabLanes - 1);
+    const int c = (blockIdx.x * kSlabLanes + l) * VEC;
+    const int t = t0 + i;
+    if (t < t_stride && c < D) {
+      Vec<VEC> r;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) r.v[k] = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) {
+        Vec<VEC> x;
+        x.load_lds(&s_red[w][i][l * VEC]);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) r.v[k] += x.v[k];
+      }
+      r.store(grad_enc + ((int64_t)(b * t_stride + t) * D + c));
+    }
+  }
+}
+
+// grad_dec[b,u,:] = sum over the frame tiles of utterance b, in tile order;
+// zero for the padding positions u > U_b.
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void joiner_dec_reduce_kernel(
+    const float *__restrict__ dec_partial, const int32_t *__restrict__ logit_lengths,
+    const int32_t *__restrict__ target_lengths, int N, int t_stride, int u_stride, int D,
+    int ntiles, float *__restrict__ grad_dec) {
+  const int nvec = D / VEC;
+  const int64_t unit = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t total = (int64_t)N * u_stride * nvec;
+  if (unit >= total) return;
+  const int c = (int)(unit % nvec) * VEC;
+  const int64_t bu = unit / nvec;
+  const int u = (int)(bu % u_stride), b = (int)(bu / u_stride);
+  Vec<VEC> r;
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) r.v[k] = 0.f;
+  if (u <= target_lengths[b]) {
+    const int T = min(logit_lengths[b], t_stride);
+    const int used = (T + kTileFrames - 1) / kTileFrames;
+    for (int tile = 0; tile < used; ++tile) {
+      Vec<VEC> x;
+      x.load_cached(dec_partial + ((((int64_t)b * ntiles + tile) * u_stride + u) * D + c));
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) r.v[k] += x.v[k];
+    }
+  }
+  r.store(grad_dec + (bu * D + c));
+}
+
+static inline int launch_status() { return (int)hipGetLastError(); }
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+static inline bool aligned4(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 3) == 0; }
+
+}  // namespace ot
+
+using namespace ot;
+
+extern "C" {
+
+int ot_joiner_rows(const int32_t *logit_lengths, const int32_t *target_lengths,
+                   const int32_t *row_splits, int32_t N, int64_t rows, int32_t t_stride,
+                   int32_t u_stride, int32_t *row_index, void *stream) {
+  if (!logit_lengths || !target_lengths || !row_splits || !row_index || N <= 0 || rows < 0 ||
+      rows > INT32_MAX || t_stride <= 0 || u_stride <= 0 ||
+      (int64_t)N * t_stride > INT32_MAX || (int64_t)N * u_stride > INT32_MAX)
+    return OT_E_BAD_ARG;
+  if (reinterpret_cast<uintptr_t>(row_index) & 7) return OT_E_MISALIGNED;
+  if (rows == 0) return 0;
+  const unsigned blocks = (unsigned)((rows + kBlock - 1) / kBlock);
+  hipLaunchKernelGGL(joiner_rows_kernel, dim3(blocks), dim3(kBlock), 0,
+                     static_cast<hipStream_t>(stream), logit_lengths, target_lengths, row_splits,
+                     N, rows, t_stride, u_stride, reinterpret_cast<int2 *>(row_index));
+  return launch_status();
+}
+
+int ot_joiner_pack(const float *enc, const float *dec, const int32_t *row_index, int64_t rows,
+                   int32_t D, int32_t activation, float *out, void *stream) {
+  if (!enc || !dec || !row_index || !out || rows < 0 || rows > INT32_MAX || D <= 0 ||
+      (activation != OT_ACT_NONE && activation != OT_ACT_TANH))
+    return OT_E_BAD_ARG;
+  if (!aligned4(enc) || !aligned4(dec) || !aligned4(out) ||
+      (reinterpret_cast<uintptr_t>(row_index) & 7))
+    return OT_E_MISALIGNED;
+  if (rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int vec = (D % 4 == 0 && aligned16(enc) && aligned16(dec) && aligned16(out)) ? 4 : 1;
+  const int nvec = D / vec;
+  const int64_t nunits = rows * nvec;
+  const int64_t per_block = (int64_t)kPackUnroll * kBlock;
+  const int64_t blocks = (nunits + per_block - 1) / per_block;
+  if (blocks > INT32_MAX) return OT_E_BAD_ARG;
+  const int2 *idx = reinterpret_cast<const int2 *>(row_index);
+#define OT_LAUNCH_PACK(VEC_, ACT_)                                                             \
+  hipLaunchKernelGGL((joiner_pack_kernel<VEC_, ACT_>), dim3((unsigned)blocks), dim3(kBlock), 0, \
+                     s, enc, dec, idx, out, nunits, nvec, 1.0f / (float)nvec, 1.0 / (double)nvec)
+  if (activation == OT_ACT_TANH) {
+    if (vec == 4) OT_LAUNCH_PACK(4, OT_ACT_TANH); else OT_LAUNCH_PACK(1, OT_ACT_TANH);
+  } else {
+    if (vec == 4) OT_LAUNCH_PACK(4, OT_ACT_NONE); else OT_LAUNCH_PACK(1, OT_ACT_NONE);
+  }
+#undef OT_LAUNCH_PACK
+  return launch_status();
+}
+
+size_t ot_joiner_unpack_workspace_bytes(int32_t N, int32_t t_stride, int32_t u_stride, int32_t D) {
+  if (N <= 0 || t_stride <= 0 || u_stride <= 0 || D <= 0) return 0;
+  const size_t ntiles = ((size_t)t_stride + kTileFrames - 1) / kTileFrames;
+  return (size_t)N * ntiles * (size_t)u_stride * (size_t)D * sizeof(float);
+}
+
+int ot_joiner_unpack_grad(const float *grad_out, const float *enc, const float *dec,
+                          const int32_t *logit_lengths, const int32_t *target_lengths,
+                          const int32_t *row_splits, int32_t N, int32_t t_stride, int32_t u_stride,
+                          int32_t D, int32_t activation, void *workspace, size_t workspace_bytes,
+                          float *grad_enc, float *grad_dec, void *stream) {
+  if (!grad_out || !logit_lengths || !target_lengths || !row_splits || !workspace || !grad_enc ||
+      !grad_dec || N <= 0 || N > 65535 || t_stride <= 0 || u_stride <= 0 || D <= 0 ||
+      (int64_t)N * t_stride > INT32_MAX || (int64_t)N * u_stride > INT32_MAX ||
+      (activation != OT_ACT_NONE && activation != OT_ACT_TANH) ||
+      (activation != OT_ACT_NONE && (!enc || !dec)))
+    return OT_E_BAD_ARG;
+  if (workspace_bytes < ot_joiner_unpack_workspace_bytes(N, t_stride, u_stride, D))
+    return OT_E_BAD_ARG;
+  if (!aligned4(grad_out) || !aligned4(enc) || !aligned4(dec) || !aligned4(grad_enc) ||
+      !aligned4(grad_dec) || !aligned16(workspace))
+    return OT_E_MISALIGNED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool v4 = D % 4 == 0 && aligned16(grad_out) && aligned16(grad_enc) && aligned16(grad_dec) &&
+                  (activation == OT_ACT_NONE || (aligned16(enc) && aligned16(dec)));
+  const int vec = v4 ? 4 : 1;
+  const int ntiles = (t_stride + kTileFrames - 1) / kTileFrames;
+  if (ntiles > 65535) return OT_E_TOO_LONG;
+  const int slab = kSlabLanes * vec;
+  const dim3 grid((unsigned)((D + slab - 1) / slab), (unsigned)ntiles, (unsigned)N);
+  float *partial = static_cast<float *>(workspace);
+#define OT_LAUNCH_UNPACK(VEC_, ACT_)                                                          \
+  hipLaunchKernelGGL((joiner_unpack_grad_kernel<VEC_, ACT_>), grid, dim3(kBlock), 0, s,       \
+                     grad_out, enc, dec, logit_lengths, target_lengths, row_splits, t_stride, \
+                     u_stride, D, grad_enc, partial)
+  if (activation == OT_ACT_TANH) {
+    if (vec == 4) OT_LAUNCH_UNPACK(4, OT_ACT_TANH); else OT_LAUNCH_UNPACK(1, OT_ACT_TANH);
+  } else {
+    if (vec == 4) OT_LAUNCH_UNPACK(4, OT_ACT_NONE); else OT_LAUNCH_UNPACK(1, OT_ACT_NONE);
+  }
+#undef OT_LAUNCH_UNPACK
+  int rc = launch_status();
+  if (rc) return rc;
+  const int64_t units = (int64_t)N * u_stride * (D / vec);
+  const int64_t blocks = (units + kBlock - 1) / kBlock;
+  if (blocks > INT32_MAX) return OT_E_BAD_ARG;
+  if (vec == 4)
+    hipLaunchKernelGGL(joiner_dec_reduce_kernel<4>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                       partial, logit_lengths, target_lengths, N, t_stride, u_stride, D, ntiles,
+                       grad_dec);
+  else
+    hipLaunchKernelGGL(joiner_dec_reduce_kernel<1>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                       partial, logit_lengths, target_lengths, N, t_stride, u_stride, D, ntiles,
+                       grad_dec);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -7,8 +7,8 @@
 //   lse_gather_kernel     per-row logsumexp + gather     cuda.cu:427 + kernels.cu:30-60
 //   gather_kernel         gather only (log-softmax in)   kernels.cu:62-88
 //   alpha_beta_kernel     lattice DP, both directions    kernels.cu:200-313, 415-519
-//   grad_logits_kernel    gradient, logits input         kernels.cu:522-651
-//   grad_logsoftmax_kernel gradient, log-softmax input   kernels.cu:653-779
+//   row_coeff_kernel      per-row part of the gradients  kernels.cu:522-779
+//   grad_flat_kernel      (rows, V) pass of the gradients kernels.cu:522-779
 //   scale_kernel          grad *= loss_grad              transducer_loss.py:162
 //
 // The two kernels that move (rows, V) data are HBM-bound streaming kernels: a

@@ -1,0 +1,80 @@
+"""Packed joiner input for :func:`transducer_loss`.
+
+The loss expects the joiner output for the valid ``(t, u)`` cells only, all
+utterances concatenated, and the reference shows how to build the joiner's
+input in that layout with Python lists (README.md:166-177)::
+
+    encoder_out_list = [encoder_out[i, :logit_lengths[i], :] for i in range(N)]
+    decoder_out_list = [decoder_out[i, :target_lengths[i]+1, :] for i in range(N)]
+    x = [e.unsqueeze(1) + d.unsqueeze(0) for e, d in zip(encoder_out_list, decoder_out_list)]
+    x = [p.reshape(-1, D) for p in x]
+    x = torch.cat(x)
+    activation = torch.tanh(x)
+
+:func:`pack_joiner` computes ``x`` (``activation=None``) or ``tanh(x)``
+(``activation="tanh"``) with one kernel, and its gradient with one pass over the
+incoming gradient.
+"""
+from typing import Optional
+
+import torch
+
+from . import _optimized_transducer
+
+
+class PackJoinerFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, encoder_out, decoder_out, logit_lengths, target_lengths, activation):
+        out, row_splits, _ = _optimized_transducer.joiner_pack(
+            encoder_out=encoder_out,
+            decoder_out=decoder_out,
+            logit_lengths=logit_lengths,
+            target_lengths=target_lengths,
+            activation=activation,
+        )
+        ctx.activation = activation
+        ctx.save_for_backward(encoder_out, decoder_out, logit_lengths, target_lengths, row_splits)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        encoder_out, decoder_out, logit_lengths, target_lengths, row_splits = ctx.saved_tensors
+        grad_enc, grad_dec = _optimized_transducer.joiner_unpack_grad(
+            grad_out=grad_out.contiguous(),
+            encoder_out=encoder_out,
+            decoder_out=decoder_out,
+            logit_lengths=logit_lengths,
+            target_lengths=target_lengths,
+            row_splits=row_splits,
+            activation=ctx.activation,
+        )
+        return grad_enc, grad_dec, None, None, None
+
+
+def pack_joiner(
+    encoder_out: torch.Tensor,
+    decoder_out: torch.Tensor,
+    logit_lengths: torch.Tensor,
+    target_lengths: torch.Tensor,
+    activation: Optional[str] = None,
+) -> torch.Tensor:
+    """Joiner input in the packed row order of :func:`transducer_loss`.
+
+    Args:
+      encoder_out: (N, T, D) float32, contiguous, on a HIP device; frames at or
+        beyond ``logit_lengths[i]`` are padding.
+      decoder_out: (N, U + 1, D) float32, output of the prediction network for
+        the blank-prepended targets; positions beyond ``target_lengths[i]`` are
+        padding.
+      logit_lengths: (N,) int32, T_i (1 <= T_i <= T).
+      target_lengths: (N,) int32, U_i (0 <= U_i <= U).
+      activation: None / "none" for ``enc + dec``, "tanh" for ``tanh(enc + dec)``.
+    Returns:
+      (sum_i T_i * (U_i + 1), D) float32: row ``row_splits[i] + t * (U_i + 1) + u``
+      holds ``act(encoder_out[i, t] + decoder_out[i, u])``.  Differentiable with
+      respect to ``encoder_out`` and ``decoder_out`` (padding gets zero gradient).
+    """
+    return PackJoinerFunction.apply(
+        encoder_out, decoder_out, logit_lengths, target_lengths,
+        "none" if activation is None else activation,
+    )

@@ -177,3 +177,50 @@ def transducer_loss(logits, targets, logit_lengths, target_lengths, blank, from_
         loss = loss.sum(dtype=dtype)
     grad *= real(loss_grad)
     return loss, grad
+
+
+# ---------------------------------------------------------------- packed joiner input
+def pack_joiner(encoder_out, decoder_out, logit_lengths, target_lengths, activation=None,
+                dtype=np.float32):
+    """The reference's recipe for the joiner input (README.md:166-177), literally:
+    per utterance e[:T, None, :] + d[None, :U+1, :], reshaped to (T*(U+1), D),
+    concatenated; then tanh when activation == "tanh"."""
+    enc = np.asarray(encoder_out, dtype=dtype)
+    dec = np.asarray(decoder_out, dtype=dtype)
+    D = enc.shape[2]
+    parts = []
+    for i in range(enc.shape[0]):
+        e = enc[i, :int(logit_lengths[i]), :]
+        d = dec[i, :int(target_lengths[i]) + 1, :]
+        parts.append((e[:, None, :] + d[None, :, :]).reshape(-1, D))
+    x = np.concatenate(parts)
+    return np.tanh(x) if activation == "tanh" else x
+
+
+def pack_joiner_backward(grad_out, encoder_out, decoder_out, logit_lengths, target_lengths,
+                         activation=None, dtype=np.float64):
+    """Gradient of pack_joiner by the chain rule: the incoming gradient of a row,
+    times 1 - tanh^2 for "tanh", is added to its encoder frame and to its decoder
+    position; padding receives zero.  Returns (grad_enc, grad_dec, abs_enc, abs_dec):
+    the last two are the same sums over the absolute values of the incoming
+    gradient, the scale of the rounding error of a float32 evaluation (of the
+    summation in any order, and of 1 - tanh^2 where tanh is close to 1)."""
+    enc = np.asarray(encoder_out, dtype=dtype)
+    dec = np.asarray(decoder_out, dtype=dtype)
+    g = np.asarray(grad_out, dtype=dtype)
+    ge, gd = np.zeros_like(enc), np.zeros_like(dec)
+    ae, ad = np.zeros_like(enc), np.zeros_like(dec)
+    D = enc.shape[2]
+    r = 0
+    for i in range(enc.shape[0]):
+        T, U1 = int(logit_lengths[i]), int(target_lengths[i]) + 1
+        gi = g[r:r + T * U1].reshape(T, U1, D)
+        ae[i, :T] = np.abs(gi).sum(1)
+        ad[i, :U1] = np.abs(gi).sum(0)
+        if activation == "tanh":
+            a = np.tanh(enc[i, :T, None, :] + dec[i, None, :U1, :])
+            gi = gi * (1.0 - a * a)
+        ge[i, :T] = gi.sum(1)
+        gd[i, :U1] = gi.sum(0)
+        r += T * U1
+    return ge, gd, ae, ad

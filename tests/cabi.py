@@ -152,3 +152,38 @@ def scale_by_device_scalar(x, factor):
 
 def copy_floats(src, dst):
     check(lib().ot_copy_floats(ptr(src), ptr(dst), ctypes.c_int64(src.numel()), stream()))
+
+
+def joiner_rows(T, U, splits, rows, t_stride, u_stride):
+    idx = torch.full((rows, 2), -7, dtype=torch.int32, device=T.device)
+    check(lib().ot_joiner_rows(ptr(T), ptr(U), ptr(splits), ctypes.c_int32(T.numel()),
+                               ctypes.c_int64(rows), ctypes.c_int32(t_stride),
+                               ctypes.c_int32(u_stride), ptr(idx), stream()))
+    return idx
+
+
+def joiner_pack(enc, dec, row_index, activation, out=None):
+    rows, D = row_index.shape[0], enc.shape[-1]
+    if out is None:
+        out = torch.full((rows, D), float("nan"), dtype=torch.float32, device=enc.device)
+    check(lib().ot_joiner_pack(ptr(enc), ptr(dec), ptr(row_index), ctypes.c_int64(rows),
+                               ctypes.c_int32(D), ctypes.c_int32(activation), ptr(out), stream()))
+    return out
+
+
+def joiner_unpack_grad(grad_out, enc, dec, T, U, splits, activation):
+    N, t_stride, D = enc.shape
+    u_stride = dec.shape[1]
+    L = lib()
+    L.ot_joiner_unpack_workspace_bytes.restype = ctypes.c_size_t
+    nbytes = L.ot_joiner_unpack_workspace_bytes(ctypes.c_int32(N), ctypes.c_int32(t_stride),
+                                                ctypes.c_int32(u_stride), ctypes.c_int32(D))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=enc.device)
+    ge = torch.full_like(enc, float("nan"))
+    gd = torch.full_like(dec, float("nan"))
+    check(L.ot_joiner_unpack_grad(ptr(grad_out), ptr(enc), ptr(dec), ptr(T), ptr(U), ptr(splits),
+                                  ctypes.c_int32(N), ctypes.c_int32(t_stride),
+                                  ctypes.c_int32(u_stride), ctypes.c_int32(D),
+                                  ctypes.c_int32(activation), ptr(ws), ctypes.c_size_t(nbytes),
+                                  ptr(ge), ptr(gd), stream()))
+    return ge, gd

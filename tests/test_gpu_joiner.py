@@ -1,0 +1,169 @@
+"""GPU parity of the packed joiner input (the data format on the input side of
+the loss): C ABI and Python entry point against the numpy restatement of the
+reference's README.md:166-177 recipe and the closed-form gradient.
+
+Tolerances.  Forward: one addition (and one tanh); |delta| <= 1e-6 + 1e-6 |ref|
+for tanh, bit-exact without activation.  Gradient: each output is a sum of up to
+max(T, U+1) float32 terms g * (1 - tanh^2); the bound is 1e-5 relative plus 1e-6
+times the sum of |g| over the same cells (a float32 sum in any order errs by at
+most eps times that sum times the number of terms, and 1 - tanh^2 carries an
+absolute error of about eps where tanh is close to 1)."""
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+import cabi
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+ACT = {None: 0, "tanh": 1}
+
+
+def _dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def _batch(rng, N, Tm, U1m, D, pad_t=0, pad_u=0):
+    T = rng.integers(1, Tm + 1, size=N).astype(np.int32)
+    U = rng.integers(0, U1m, size=N).astype(np.int32)
+    T[0], U[0] = 1, 0
+    if N > 1:
+        T[1], U[1] = Tm, U1m - 1
+    if N > 2:
+        T[2], U[2] = 1, U1m - 1
+    enc = rng.standard_normal((N, Tm + pad_t, D)).astype(np.float32)
+    dec = rng.standard_normal((N, U1m + pad_u, D)).astype(np.float32)
+    return T, U, enc, dec
+
+
+CASES = [  # name, N, Tmax, U1max, D, pad_t, pad_u
+    ("small_D8", 4, 9, 5, 8, 0, 0),
+    ("D7_scalar_path", 5, 20, 6, 7, 2, 1),
+    ("D64_one_slab", 6, 37, 19, 64, 0, 3),
+    ("D100_partial_slab", 3, 50, 33, 100, 5, 0),
+    ("D512_long_T", 3, 130, 40, 512, 0, 0),
+    ("many_utts", 70, 6, 4, 16, 1, 1),
+]
+
+
+@pytest.mark.parametrize("activation", [None, "tanh"])
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_pack_and_unpack_through_the_c_abi(case, activation, device):
+    _, N, Tm, U1m, D, pad_t, pad_u = case
+    rng = np.random.default_rng(zlib.crc32(case[0].encode()))
+    T, U, enc, dec = _batch(rng, N, Tm, U1m, D, pad_t, pad_u)
+    dT, dU, denc, ddec = _dev(T, device), _dev(U, device), _dev(enc, device), _dev(dec, device)
+    splits, st = cabi.row_splits(dT, dU, torch.zeros((N, 0), dtype=torch.int32, device=device))
+    rows = int(st.sum_tu)
+    want = oracle.pack_joiner(enc, dec, T, U, activation)
+    assert want.shape == (rows, D)
+
+    # row -> (encoder frame, decoder position): integers, bit exact
+    idx = cabi.joiner_rows(dT, dU, splits, rows, enc.shape[1], dec.shape[1]).cpu().numpy()
+    sp, _ = oracle.row_splits(T, U)
+    ids = oracle.row_ids(sp)
+    local = np.arange(rows) - sp[ids]
+    t, u = local // (U[ids] + 1), local % (U[ids] + 1)
+    assert (idx[:, 0] == ids * enc.shape[1] + t).all() and (idx[:, 1] == ids * dec.shape[1] + u).all()
+
+    out = cabi.joiner_pack(denc, ddec, _dev(idx, device), ACT[activation]).cpu().numpy()
+    if activation is None:
+        assert (out == want).all()
+    else:
+        assert np.allclose(out, want, rtol=1e-6, atol=1e-6), np.abs(out - want).max()
+
+    g = rng.standard_normal((rows, D)).astype(np.float32)
+    ge, gd = cabi.joiner_unpack_grad(_dev(g, device), denc, ddec, dT, dU, splits, ACT[activation])
+    ge, gd = ge.cpu().numpy(), gd.cpu().numpy()
+    we, wd, ae, ad = oracle.pack_joiner_backward(g, enc, dec, T, U, activation)
+    assert not np.isnan(ge).any() and not np.isnan(gd).any()  # written in full, padding included
+    assert (np.abs(ge - we) <= 1e-5 * np.abs(we) + 1e-6 * ae + 1e-30).all(), np.abs(ge - we).max()
+    assert (np.abs(gd - wd) <= 1e-5 * np.abs(wd) + 1e-6 * ad + 1e-30).all(), np.abs(gd - wd).max()
+    for b in range(N):  # padding is exactly zero
+        assert (ge[b, T[b]:] == 0).all() and (gd[b, U[b] + 1:] == 0).all()
+    # fixed summation order: same bits on a second run
+    ge2, gd2 = cabi.joiner_unpack_grad(_dev(g, device), denc, ddec, dT, dU, splits, ACT[activation])
+    assert (ge2.cpu().numpy() == ge).all() and (gd2.cpu().numpy() == gd).all()
+
+
+def test_tanh_accuracy_over_the_whole_range(device):
+    # enc = x, dec = 0: out = tanh(x); relative error of a few ulp everywhere (8 allowed)
+    x = np.concatenate([np.linspace(-12, 12, 4001), np.array([0.0, 1e-8, -1e-8, 1e-4, 0.2499, 0.25,
+                       0.2501, 20.0, -20.0, 100.0, -100.0])]).astype(np.float32)
+    n = x.size
+    pad = (-n) % 4
+    x = np.concatenate([x, np.zeros(pad, np.float32)])
+    enc = x.reshape(1, 1, -1)
+    dec = np.zeros_like(enc)
+    T, U = np.array([1], np.int32), np.array([0], np.int32)
+    dT, dU = _dev(T, device), _dev(U, device)
+    splits, _ = cabi.row_splits(dT, dU, torch.zeros((1, 0), dtype=torch.int32, device=device))
+    idx = cabi.joiner_rows(dT, dU, splits, 1, 1, 1)
+    out = cabi.joiner_pack(_dev(enc, device), _dev(dec, device), idx, 1).cpu().numpy()[0]
+    want = np.tanh(x.astype(np.float64))
+    assert (np.abs(out - want) <= 8 * np.spacing(np.abs(want).astype(np.float32)) + 1e-45).all()
+    assert (np.sign(out) == np.sign(want)).all() and np.abs(out).max() <= 1.0
+
+
+@pytest.mark.parametrize("activation", [None, "tanh"])
+def test_python_entry_point_and_autograd(activation, device):
+    import optimized_transducer_amd as ot
+    rng = np.random.default_rng(3)
+    T, U, enc, dec = _batch(rng, 6, 25, 9, 48, pad_t=3, pad_u=2)
+    dT, dU = _dev(T, device), _dev(U, device)
+    te = _dev(enc, device).requires_grad_(True)
+    td = _dev(dec, device).requires_grad_(True)
+    x = ot.pack_joiner(te, td, dT, dU, activation=activation)
+    want = oracle.pack_joiner(enc, dec, T, U, activation)
+    assert x.shape == want.shape and np.allclose(x.detach().cpu().numpy(), want, rtol=1e-6, atol=1e-6)
+    # the README.md:166-177 recipe in torch on the device gives the same numbers and gradients
+    re = _dev(enc, device).requires_grad_(True)
+    rd = _dev(dec, device).requires_grad_(True)
+    parts = [(re[i, :T[i]].unsqueeze(1) + rd[i, :U[i] + 1].unsqueeze(0)).reshape(-1, 48)
+             for i in range(6)]
+    y = torch.cat(parts)
+    if activation == "tanh":
+        y = torch.tanh(y)
+    assert torch.allclose(x, y, rtol=1e-6, atol=1e-6)
+    g = torch.randn_like(x)
+    x.backward(g)
+    y.backward(g)
+    assert torch.allclose(te.grad, re.grad, rtol=1e-4, atol=1e-5)
+    assert torch.allclose(td.grad, rd.grad, rtol=1e-4, atol=1e-5)
+
+    # end to end: joiner -> Linear -> transducer loss, gradients reach encoder and decoder
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(48, 20).to(device)
+    tg = _dev(rng.integers(1, 20, size=(6, int(U.max()))).astype(np.int32), device)
+    te.grad = td.grad = None
+    loss = ot.transducer_loss(lin(ot.pack_joiner(te, td, dT, dU, activation="tanh")), tg, dT, dU, 0,
+                              False, reduction="sum")
+    loss.backward()
+    assert torch.isfinite(loss) and te.grad.abs().sum() > 0 and td.grad.abs().sum() > 0
+    assert (te.grad[0, T[0]:] == 0).all()
+
+
+def test_argument_checks(device):
+    import optimized_transducer_amd as ot
+    rng = np.random.default_rng(4)
+    T, U, enc, dec = _batch(rng, 3, 8, 4, 8)
+    dT, dU, de, dd = _dev(T, device), _dev(U, device), _dev(enc, device), _dev(dec, device)
+    with pytest.raises(RuntimeError, match="logit_lengths.max"):
+        ot.pack_joiner(de[:, :5].contiguous(), dd, dT, dU)
+    with pytest.raises(RuntimeError, match="target_lengths.max"):
+        ot.pack_joiner(de, dd[:, :2].contiguous(), dT, dU)
+    with pytest.raises(RuntimeError, match="last dimension"):
+        ot.pack_joiner(de, dd[:, :, :4].contiguous(), dT, dU)
+    with pytest.raises(RuntimeError, match="activation"):
+        ot.pack_joiner(de, dd, dT, dU, activation="relu")
+    with pytest.raises(RuntimeError, match="no CPU"):
+        ot.pack_joiner(torch.from_numpy(enc), torch.from_numpy(dec), torch.from_numpy(T),
+                       torch.from_numpy(U))
+    bad = T.copy()
+    bad[1] = 0
+    with pytest.raises(RuntimeError, match="logit_lengths >= 1"):
+        ot.pack_joiner(de, dd, _dev(bad, device), dU)
+    assert ot.pack_joiner(de, dd, dT, dU).shape == (int((T * (U + 1)).sum()), 8)

@@ -353,3 +353,50 @@ def test_oracle_against_compiled_reference_live(fls, one_sym):
                                                    in_place=True)
             assert g2 is buf and (buf == g).all()
             assert wg.ctypes.data == xt.detach().numpy().ctypes.data  # the reference aliases too
+
+
+# ------------------------------------------------------------ packed joiner input
+def _readme_joiner(encoder_out, decoder_out, logit_lengths, target_lengths, tanh):
+    # the reference's usage recipe, README.md:166-177, in torch (float64, autograd)
+    N, D = encoder_out.shape[0], encoder_out.shape[2]
+    encoder_out_list = [encoder_out[i, :logit_lengths[i], :] for i in range(N)]
+    decoder_out_list = [decoder_out[i, :target_lengths[i] + 1, :] for i in range(N)]
+    x = [e.unsqueeze(1) + d.unsqueeze(0) for e, d in zip(encoder_out_list, decoder_out_list)]
+    x = [p.reshape(-1, D) for p in x]
+    x = torch.cat(x)
+    return torch.tanh(x) if tanh else x
+
+
+@pytest.mark.parametrize("activation", [None, "tanh"])
+def test_pack_joiner_oracle_matches_the_readme_recipe_and_its_autograd(activation):
+    rng = np.random.default_rng(11)
+    N, Tm, Um, D = 5, 9, 6, 7
+    T = rng.integers(1, Tm + 1, size=N).astype(np.int32)
+    U = rng.integers(0, Um, size=N).astype(np.int32)
+    T[0], U[0] = 1, 0
+    T[1], U[1] = Tm, Um - 1
+    enc = rng.standard_normal((N, Tm, D))
+    dec = rng.standard_normal((N, Um, D))
+    te = torch.tensor(enc, requires_grad=True)
+    td = torch.tensor(dec, requires_grad=True)
+    want = _readme_joiner(te, td, T.tolist(), U.tolist(), activation == "tanh")
+    got = oracle.pack_joiner(enc, dec, T, U, activation, dtype=np.float64)
+    assert got.shape == tuple(want.shape) == (int((T * (U + 1)).sum()), D)
+    assert np.allclose(got, want.detach().numpy(), rtol=1e-14, atol=1e-14)
+    # row order is the packed order of the loss: row_splits[b] + t*(U_b+1) + u
+    splits, _ = oracle.row_splits(T, U)
+    b, t, u = 1, 3, 2
+    row = splits[b] + t * (U[b] + 1) + u
+    s = enc[b, t] + dec[b, u]
+    assert np.allclose(got[row], np.tanh(s) if activation == "tanh" else s)
+    g = rng.standard_normal(got.shape)
+    want.backward(torch.tensor(g))
+    ge, gd, ae, ad = oracle.pack_joiner_backward(g, enc, dec, T, U, activation)
+    assert np.allclose(ge, te.grad.numpy(), rtol=1e-12, atol=1e-12)
+    assert np.allclose(gd, td.grad.numpy(), rtol=1e-12, atol=1e-12)
+    assert (ge[0, 1:] == 0).all() and (gd[0, 1:] == 0).all()  # padding
+    assert (ae >= np.abs(ge) - 1e-12).all() and (ad >= np.abs(gd) - 1e-12).all()
+    assert np.isclose(ae.sum(), np.abs(g).sum()) and np.isclose(ad.sum(), np.abs(g).sum())
+    # float32 evaluation of the forward agrees with float64 to rounding
+    got32 = oracle.pack_joiner(enc.astype(np.float32), dec.astype(np.float32), T, U, activation)
+    assert got32.dtype == np.float32 and np.allclose(got32, got, rtol=1e-6, atol=1e-6)
