@@ -104,6 +104,93 @@ def cpu_baseline(w, logits_host, max_seconds=30.0):
     }
 
 
+def bench_joiner(args):
+    """Secondary benchmark: the packed joiner input (pack_joiner, tanh) forward +
+    backward for the lengths of the chosen workload; not the headline metric."""
+    import numpy as np
+    import torch
+    import optimized_transducer_amd as ot
+    from optimized_transducer_amd import _optimized_transducer as ext
+
+    dev = torch.device("cuda", 0)
+    w = make_workload(args.workload)
+    K, W, D = args.steps, args.warmup, args.joiner_dim
+    N, R = w.N, w.rows
+    Tm, U1m = int(w.logit_lengths.max()), int(w.target_lengths.max()) + 1
+    gen = torch.Generator(device="cpu").manual_seed(w.seed)
+    enc_h = torch.randn((N, Tm, D), generator=gen)
+    dec_h = torch.randn((N, U1m, D), generator=gen)
+    enc = enc_h.to(dev).requires_grad_(True)
+    dec = dec_h.to(dev).requires_grad_(True)
+    T = torch.from_numpy(w.logit_lengths).to(dev)
+    U = torch.from_numpy(w.target_lengths).to(dev)
+    g = torch.randn((R, D), device=dev)
+
+    def step():
+        enc.grad = dec.grad = None
+        x = ot.pack_joiner(enc, dec, T, U, activation="tanh")
+        x.backward(g)
+
+    for _ in range(W):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    out = {
+        "metric": "utterances/sec packed joiner input (tanh) fwd+bwd; achieved HBM GB/s vs peak",
+        "value": N * K / elapsed, "unit": "utterances/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": 1e3 * elapsed / K, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "joiner_input_of_" + w.name, "N": N, "D": D, "packed_rows": R,
+                   "T_max": Tm, "U1_max": U1m, "activation": "tanh", "packed_bytes": 4 * R * D},
+    }
+    ext.set_profiling(True)
+    for _ in range(K):
+        step()
+    torch.cuda.synchronize()
+    ext.set_profiling(False)
+    per = {}
+    for name, ms in ext.take_profile():
+        per.setdefault(name, []).append(ms)
+    # pack: writes (rows, D) once; unpack: reads (rows, D) once and
+    # writes + re-reads one partial decoder sum per 16 frames
+    alg = {"joiner_pack": 4 * D * R, "joiner_unpack_grad": 4 * D * R + 2 * (4 * D * R // 16)}
+    kernels = {}
+    for name, ms in per.items():
+        per_step = sum(ms) / K
+        kernels[name] = {"ms_per_step": per_step, "launches_per_step": len(ms) / K}
+        if name in alg:
+            kernels[name]["algorithmic_bytes"] = alg[name]
+            kernels[name]["achieved_GBps"] = alg[name] / (per_step * 1e-3) / 1e9
+    dom = max(alg, key=lambda k: kernels[k]["ms_per_step"])
+    out["roofline"] = {"bound": "hbm", "kernel": dom + "_kernel", "peak": HBM_PEAK_GBPS,
+                       "achieved": kernels[dom]["achieved_GBps"], "unit": "GB/s",
+                       "frac": kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, "traffic": None,
+                       "kernel_ms_per_step": kernels[dom]["ms_per_step"],
+                       "algorithmic_bytes_per_step": alg[dom]}
+    out["kernels"] = kernels
+    if not args.no_cpu_baseline:
+        # the reference's own recipe (README.md:166-177) in torch on the host cores
+        e = enc_h.clone().requires_grad_(True)
+        d = dec_h.clone().requires_grad_(True)
+        gh = g.cpu()
+        Tl, Ul = w.logit_lengths.tolist(), w.target_lengths.tolist()
+        t0 = time.perf_counter()
+        parts = [(e[i, :Tl[i]].unsqueeze(1) + d[i, :Ul[i] + 1].unsqueeze(0)).reshape(-1, D)
+                 for i in range(N)]
+        torch.tanh(torch.cat(parts)).backward(gh)
+        sec = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": N / sec, "unit": "utterances/s",
+                               "cores": torch.get_num_threads(), "kind": "reference",
+                               "sample": "one full batch: the README.md:166-177 recipe "
+                                         "(list of slices, cat, tanh) and its autograd in torch",
+                               "seconds_per_batch": sec}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -115,6 +202,10 @@ def main():
     ap.add_argument("--loss-weight", type=float, default=1.0,
                     help="multiply the loss by this before backward (a weighted or scaled loss); "
                          "the headline figure uses 1")
+    ap.add_argument("--op", default="loss", choices=["loss", "joiner"],
+                    help="loss: the headline benchmark; joiner: the packed joiner input "
+                         "(pack_joiner) forward + backward for the workload's lengths")
+    ap.add_argument("--joiner-dim", type=int, default=512)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -132,6 +223,8 @@ def main():
     from optimized_transducer_amd import _optimized_transducer as ext
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.op == "joiner":
+        return bench_joiner(args)
     dev = torch.device("cuda", 0)
     w = make_workload(args.workload)
     K, W = args.steps, args.warmup

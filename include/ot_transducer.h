@@ -235,19 +235,15 @@ int ot_transducer_loss(const float *logits, const int32_t *targets,
 #define OT_ACT_TANH 1 /* out = tanh(enc + dec)                                */
 #define OT_JOINER_TILE_FRAMES 16 /* frames per partial decoder sum            */
 
-/* row_index: (rows, 2) int32, 8-byte aligned: for packed row r of utterance b,
- * cell (t, u): {b*t_stride + t, b*u_stride + u}, the source rows in enc and
- * dec viewed as (N*t_stride, D) and (N*u_stride, D); {-1, -1} for rows beyond
- * row_splits[N].  Depends on the lengths only: compute once per batch. */
-int ot_joiner_rows(const int32_t *logit_lengths, const int32_t *target_lengths,
-                   const int32_t *row_splits, int32_t N, int64_t rows,
-                   int32_t t_stride, int32_t u_stride, int32_t *row_index,
-                   void *stream);
-
-/* out (rows, D): out[r] = act(enc[row_index[r][0]] + dec[row_index[r][1]]);
- * one streaming pass, 4*D bytes written per row. */
-int ot_joiner_pack(const float *enc, const float *dec, const int32_t *row_index,
-                   int64_t rows, int32_t D, int32_t activation, float *out,
+/* out (rows, D), rows = row_splits[N]: for utterance b and cell (t, u),
+ *   out[row_splits[b] + t*(U_b+1) + u] = act(enc[b,t] + dec[b,u]);
+ * one streaming pass, 4*D bytes written per row.  Lengths beyond the strides
+ * are clamped (nothing is read outside enc and dec); it is the caller's
+ * business that `out` holds row_splits[N] rows. */
+int ot_joiner_pack(const float *enc, const float *dec,
+                   const int32_t *logit_lengths, const int32_t *target_lengths,
+                   const int32_t *row_splits, int32_t N, int32_t t_stride,
+                   int32_t u_stride, int32_t D, int32_t activation, float *out,
                    void *stream);
 
 /* Gradient of ot_joiner_pack: given grad_out (rows, D) = d loss / d out,

@@ -477,8 +477,8 @@ void check_joiner_inputs(const torch::Tensor &enc, const torch::Tensor &dec,
               "pack_joiner: tensor sizes out of range");
 }
 
-// (packed (rows, D), row_splits (N+1) int32, row_index (rows, 2) int32)
-std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> joiner_pack(
+// (packed (rows, D), row_splits (N+1) int32)
+std::pair<torch::Tensor, torch::Tensor> joiner_pack(
     const torch::Tensor &enc, const torch::Tensor &dec, const torch::Tensor &logit_lengths,
     const torch::Tensor &target_lengths, const std::string &activation) {
   const int act = activation_code(activation);
@@ -514,21 +514,15 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> joiner_pack(
   TORCH_CHECK(rows > 0 && rows <= INT32_MAX, "pack_joiner: sum of T * (U + 1) is ", rows,
               ", outside (0, 2^31)");
 
-  torch::Tensor row_index = torch::empty({rows, 2}, logit_lengths.options());
   torch::Tensor out = torch::empty({rows, D}, enc.options());
-  {
-    ScopedTimer timer("joiner_rows", stream);
-    OT_CHECK(ot_joiner_rows(logit_lengths.data_ptr<int32_t>(), target_lengths.data_ptr<int32_t>(),
-                            row_splits.data_ptr<int32_t>(), (int32_t)N, rows, (int32_t)Tmax,
-                            (int32_t)U1max, row_index.data_ptr<int32_t>(), stream));
-  }
   {
     ScopedTimer timer("joiner_pack", stream);
     OT_CHECK(ot_joiner_pack(enc.data_ptr<float>(), dec.data_ptr<float>(),
-                            row_index.data_ptr<int32_t>(), rows, (int32_t)D, act,
-                            out.data_ptr<float>(), stream));
+                            logit_lengths.data_ptr<int32_t>(), target_lengths.data_ptr<int32_t>(),
+                            row_splits.data_ptr<int32_t>(), (int32_t)N, (int32_t)Tmax,
+                            (int32_t)U1max, (int32_t)D, act, out.data_ptr<float>(), stream));
   }
-  return {out, row_splits, row_index};
+  return {out, row_splits};
 }
 
 // (grad_encoder_out (N, T, D), grad_decoder_out (N, U+1, D)) for grad_out (rows, D)
@@ -591,7 +585,7 @@ PYBIND11_MODULE(_optimized_transducer, m) {
   m.def("joiner_pack", &joiner_pack, py::arg("encoder_out"), py::arg("decoder_out"),
         py::arg("logit_lengths"), py::arg("target_lengths"), py::arg("activation"),
         "Packed joiner input act(enc[b,t] + dec[b,u]) for the valid (t, u) cells, in the row order "
-        "of the loss; returns (packed (rows, D), row_splits, row_index).");
+        "of the loss; returns (packed (rows, D), row_splits).");
   m.def("joiner_unpack_grad", &joiner_unpack_grad, py::arg("grad_out"), py::arg("encoder_out"),
         py::arg("decoder_out"), py::arg("logit_lengths"), py::arg("target_lengths"),
         py::arg("row_splits"), py::arg("activation"),

@@ -8,7 +8,6 @@
 //     activation = tanh(x)
 // The kernels here do the same from the padded encoder / decoder outputs in one
 // pass each way:
-//   joiner_rows_kernel         row -> (encoder frame, decoder position), 8 B/row
 //   joiner_pack_kernel         out[row] = act(enc[b,t] + dec[b,u]); write-bound
 //   joiner_unpack_grad_kernel  one pass over d(out): complete sums over u for
 //                              the encoder, sums over 16 frames for the decoder
@@ -51,69 +50,59 @@ __device__ __forceinline__ float activate_slope(float s) {
 }
 
 // ---------------------------------------------------------------------------
-// row -> source rows of the padded encoder / decoder outputs
+// forward
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void joiner_rows_kernel(
-    const int32_t *__restrict__ logit_lengths, const int32_t *__restrict__ target_lengths,
-    const int32_t *__restrict__ row_splits, int N, int64_t rows, int t_stride, int u_stride,
-    int2 *__restrict__ row_index) {
-  __shared__ BlockUtterances bu;
-  const int64_t row_first = (int64_t)blockIdx.x * kBlock;
-  const int64_t row_end = min(rows, row_first + kBlock);
-  bu.load(row_splits, N, row_first, row_end - 1);
-  const int64_t row = row_first + threadIdx.x;
-  if (row >= row_end) return;
-  int2 idx = make_int2(-1, -1);  // rows beyond the batch (inconsistent sizes): no source
-  if (row < (int64_t)row_splits[N]) {
-    const Cell c = decode_row(bu, row, logit_lengths, target_lengths);
-    if (c.t < t_stride && c.u < u_stride) idx = make_int2(c.b * t_stride + c.t, c.b * u_stride + c.u);
-  }
-  row_index[row] = idx;
-}
-
-// ---------------------------------------------------------------------------
-// forward: flat pass over the (rows, D) output in units of VEC floats
-// ---------------------------------------------------------------------------
-constexpr int kPackUnroll = 2;
+// One workgroup = utterance b, kPackFrames frames, all positions u,
+// up to 256 column units.  A thread keeps its columns of the frames' encoder rows
+// in registers and walks u: one decoder load serves kPackFrames output rows, no
+// index array is read, and every store instruction of a wave writes a contiguous
+// piece of one output row.
+constexpr int kPackFrames = 2;  // fastest of 1, 2, 4, 8 on MI355X
 
 template <int VEC, int ACT>
 __global__ __launch_bounds__(kBlock) void joiner_pack_kernel(
     const float *__restrict__ enc, const float *__restrict__ dec,
-    const int2 *__restrict__ row_index, float *__restrict__ out, int64_t nunits, int nvec,
-    float inv_nvec, double inv_nvec_d) {
-  const int64_t base = (int64_t)blockIdx.x * (kPackUnroll * kBlock);
-  // base / nvec through a double reciprocal (exact below 2^53) and one correction step
-  int64_t row_base = (int64_t)((double)base * inv_nvec_d);
-  {
-    const int64_t r = base - row_base * nvec;
-    if (r < 0) --row_base; else if (r >= nvec) ++row_base;
+    const int32_t *__restrict__ logit_lengths, const int32_t *__restrict__ target_lengths,
+    const int32_t *__restrict__ row_splits, int t_stride, int u_stride, int D,
+    float *__restrict__ out) {
+  const int b = blockIdx.z;
+  const int t0 = blockIdx.y * kPackFrames;
+  const int T = min(logit_lengths[b], t_stride);
+  if (t0 >= T) return;
+  const int U1 = min(target_lengths[b] + 1, u_stride);
+  const int nvec = D / VEC;
+  const int cpb = min(nvec, kBlock);  // column units per workgroup
+  const int phases = kBlock / cpb;    // positions u in flight per workgroup
+  const int phase = threadIdx.x / cpb;
+  const int unit = blockIdx.x * cpb + (threadIdx.x - phase * cpb);
+  if (phase >= phases || unit >= nvec) return;
+  const int col = unit * VEC;
+  const int nt = min(kPackFrames, T - t0);
+  Vec<VEC> e[kPackFrames];
+#pragma unroll
+  for (int i = 0; i < kPackFrames; ++i) {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) e[i].v[k] = 0.f;
+    if (i < nt) e[i].load_cached(enc + ((int64_t)(b * t_stride + t0 + i) * D + col));
   }
-  const int rem_base = (int)(base - row_base * nvec);
-  const unsigned span_bytes =
-      (unsigned)min((int64_t)(kPackUnroll * kBlock), nunits - base) * (VEC * 4u);
-  const __amdgpu_buffer_rsrc_t out_buf = make_buffer(out + base * VEC, span_bytes);
-  const int64_t last_row = (nunits - 1) / nvec;
+  float *o = out + (((int64_t)row_splits[b] + (int64_t)t0 * U1) * D + col);
+  const float *dp = dec + ((int64_t)b * u_stride * D + col);
+  const int64_t frame_stride = (int64_t)U1 * D;
+  Vec<VEC> d;
+  if (phase < U1) d.load_cached(dp + (int64_t)phase * D);
+  for (int u = phase; u < U1; u += phases) {
+    Vec<VEC> dn = d;
+    if (u + phases < U1) dn.load_cached(dp + (int64_t)(u + phases) * D);
 #pragma unroll
-  for (int k = 0; k < kPackUnroll; ++k) {
-    const int local = k * kBlock + (int)threadIdx.x;
-    const int idx = rem_base + local;  // < nvec + kPackUnroll*256: exact in float
-    int q = (int)((float)idx * inv_nvec);
-    if (q * nvec > idx) --q; else if ((q + 1) * nvec <= idx) ++q;
-    const int col = (idx - q * nvec) * VEC;
-    const int64_t row = min(row_base + q, last_row);
-    const int2 src = row_index[row];
-    Vec<VEC> y;
-    if (src.x >= 0) {
-      Vec<VEC> e, d;
-      e.load_cached(enc + ((int64_t)src.x * nvec * VEC + col));
-      d.load_cached(dec + ((int64_t)src.y * nvec * VEC + col));
+    for (int i = 0; i < kPackFrames; ++i) {
+      if (i < nt) {
+        Vec<VEC> y;
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) y.v[i] = activate<ACT>(e.v[i] + d.v[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) y.v[i] = 0.f;
+        for (int k = 0; k < VEC; ++k) y.v[k] = activate<ACT>(e[i].v[k] + d.v[k]);
+        y.store_stream(o + (i * frame_stride + (int64_t)u * D));
+      }
     }
-    y.store_buffer(out_buf, (unsigned)local * (VEC * 4u));
+    d = dn;
   }
 }
 
@@ -212,8 +201,8 @@ __global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
 #pragma unroll
     for (int k = 0; k < VEC; ++k) {
       float v = acc[i].v[k];
-      v += __shfl_xor(v, 16, kWave);
-      v += __shfl_xor(v, 32, kWave);
+      if (kSlabLanes <= 16) v += __shfl_xor(v, 16, kWave);
+      if (kSlabLanes <= 32) v += __shfl_xor(v, 32, kWave);
       acc[i].v[k] = v;
     }
   const int wave = threadIdx.x / kWave;
@@ -222,9 +211,9 @@ __global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
     for (int i = 0; i < kTileFrames; ++i) acc[i].store_lds(&s_red[wave][i][lane * VEC]);
   }
   __syncthreads();
-  // 16 frames x 16 lanes = 256 (frame, lane) pairs: one per thread
-  {
-    const int i = threadIdx.x / kSlabLanes, l = threadIdx.x & (kSlabLanes - 1);
+  // 16 frames x kSlabLanes (frame, lane) pairs over the workgroup's threads
+  for (int pair = threadIdx.x; pair < kTileFrames * kSlabLanes; pair += kBlock) {
+    const int i = pair / kSlabLanes, l = pair & (kSlabLanes - 1);
     const int c = (blockIdx.x * kSlabLanes + l) * VEC;
     const int t = t0 + i;
     if (t < t_stride && c < D) {
@@ -283,48 +272,32 @@ using namespace ot;
 
 extern "C" {
 
-int ot_joiner_rows(const int32_t *logit_lengths, const int32_t *target_lengths,
-                   const int32_t *row_splits, int32_t N, int64_t rows, int32_t t_stride,
-                   int32_t u_stride, int32_t *row_index, void *stream) {
-  if (!logit_lengths || !target_lengths || !row_splits || !row_index || N <= 0 || rows < 0 ||
-      rows > INT32_MAX || t_stride <= 0 || u_stride <= 0 ||
-      (int64_t)N * t_stride > INT32_MAX || (int64_t)N * u_stride > INT32_MAX)
-    return OT_E_BAD_ARG;
-  if (reinterpret_cast<uintptr_t>(row_index) & 7) return OT_E_MISALIGNED;
-  if (rows == 0) return 0;
-  const unsigned blocks = (unsigned)((rows + kBlock - 1) / kBlock);
-  hipLaunchKernelGGL(joiner_rows_kernel, dim3(blocks), dim3(kBlock), 0,
-                     static_cast<hipStream_t>(stream), logit_lengths, target_lengths, row_splits,
-                     N, rows, t_stride, u_stride, reinterpret_cast<int2 *>(row_index));
-  return launch_status();
-}
-
-int ot_joiner_pack(const float *enc, const float *dec, const int32_t *row_index, int64_t rows,
-                   int32_t D, int32_t activation, float *out, void *stream) {
-  if (!enc || !dec || !row_index || !out || rows < 0 || rows > INT32_MAX || D <= 0 ||
+int ot_joiner_pack(const float *enc, const float *dec, const int32_t *logit_lengths,
+                   const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
+                   int32_t t_stride, int32_t u_stride, int32_t D, int32_t activation, float *out,
+                   void *stream) {
+  if (!enc || !dec || !logit_lengths || !target_lengths || !row_splits || !out || N <= 0 ||
+      N > 65535 || t_stride <= 0 || u_stride <= 0 || D <= 0 ||
+      (int64_t)N * t_stride > INT32_MAX || (int64_t)N * u_stride > INT32_MAX ||
       (activation != OT_ACT_NONE && activation != OT_ACT_TANH))
     return OT_E_BAD_ARG;
-  if (!aligned4(enc) || !aligned4(dec) || !aligned4(out) ||
-      (reinterpret_cast<uintptr_t>(row_index) & 7))
-    return OT_E_MISALIGNED;
-  if (rows == 0) return 0;
+  if (!aligned4(enc) || !aligned4(dec) || !aligned4(out)) return OT_E_MISALIGNED;
+  if ((t_stride + kPackFrames - 1) / kPackFrames > 65535) return OT_E_TOO_LONG;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int vec = (D % 4 == 0 && aligned16(enc) && aligned16(dec) && aligned16(out)) ? 4 : 1;
   const int nvec = D / vec;
-  const int64_t nunits = rows * nvec;
-  const int64_t per_block = (int64_t)kPackUnroll * kBlock;
-  const int64_t blocks = (nunits + per_block - 1) / per_block;
-  if (blocks > INT32_MAX) return OT_E_BAD_ARG;
-  const int2 *idx = reinterpret_cast<const int2 *>(row_index);
-#define OT_LAUNCH_PACK(VEC_, ACT_)                                                             \
-  hipLaunchKernelGGL((joiner_pack_kernel<VEC_, ACT_>), dim3((unsigned)blocks), dim3(kBlock), 0, \
-                     s, enc, dec, idx, out, nunits, nvec, 1.0f / (float)nvec, 1.0 / (double)nvec)
+  const int cpb = nvec < kBlock ? nvec : kBlock;
+  const dim3 grid((unsigned)((nvec + cpb - 1) / cpb),
+                  (unsigned)((t_stride + kPackFrames - 1) / kPackFrames), (unsigned)N);
+#define OT_LAUNCH_PACKT(VEC_, ACT_)                                                             \
+  hipLaunchKernelGGL((joiner_pack_kernel<VEC_, ACT_>), grid, dim3(kBlock), 0, s, enc, dec, \
+                     logit_lengths, target_lengths, row_splits, t_stride, u_stride, D, out)
   if (activation == OT_ACT_TANH) {
-    if (vec == 4) OT_LAUNCH_PACK(4, OT_ACT_TANH); else OT_LAUNCH_PACK(1, OT_ACT_TANH);
+    if (vec == 4) OT_LAUNCH_PACKT(4, OT_ACT_TANH); else OT_LAUNCH_PACKT(1, OT_ACT_TANH);
   } else {
-    if (vec == 4) OT_LAUNCH_PACK(4, OT_ACT_NONE); else OT_LAUNCH_PACK(1, OT_ACT_NONE);
+    if (vec == 4) OT_LAUNCH_PACKT(4, OT_ACT_NONE); else OT_LAUNCH_PACKT(1, OT_ACT_NONE);
   }
-#undef OT_LAUNCH_PACK
+#undef OT_LAUNCH_PACKT
   return launch_status();
 }
 

@@ -25,7 +25,7 @@ from . import _optimized_transducer
 class PackJoinerFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, encoder_out, decoder_out, logit_lengths, target_lengths, activation):
-        out, row_splits, _ = _optimized_transducer.joiner_pack(
+        out, row_splits = _optimized_transducer.joiner_pack(
             encoder_out=encoder_out,
             decoder_out=decoder_out,
             logit_lengths=logit_lengths,

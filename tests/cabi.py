@@ -154,19 +154,11 @@ def copy_floats(src, dst):
     check(lib().ot_copy_floats(ptr(src), ptr(dst), ctypes.c_int64(src.numel()), stream()))
 
 
-def joiner_rows(T, U, splits, rows, t_stride, u_stride):
-    idx = torch.full((rows, 2), -7, dtype=torch.int32, device=T.device)
-    check(lib().ot_joiner_rows(ptr(T), ptr(U), ptr(splits), ctypes.c_int32(T.numel()),
-                               ctypes.c_int64(rows), ctypes.c_int32(t_stride),
-                               ctypes.c_int32(u_stride), ptr(idx), stream()))
-    return idx
-
-
-def joiner_pack(enc, dec, row_index, activation, out=None):
-    rows, D = row_index.shape[0], enc.shape[-1]
-    if out is None:
-        out = torch.full((rows, D), float("nan"), dtype=torch.float32, device=enc.device)
-    check(lib().ot_joiner_pack(ptr(enc), ptr(dec), ptr(row_index), ctypes.c_int64(rows),
+def joiner_pack(enc, dec, T, U, splits, rows, activation):
+    N, t_stride, D = enc.shape
+    out = torch.full((rows, D), float("nan"), dtype=torch.float32, device=enc.device)
+    check(lib().ot_joiner_pack(ptr(enc), ptr(dec), ptr(T), ptr(U), ptr(splits), ctypes.c_int32(N),
+                               ctypes.c_int32(t_stride), ctypes.c_int32(dec.shape[1]),
                                ctypes.c_int32(D), ctypes.c_int32(activation), ptr(out), stream()))
     return out
 
