@@ -43,8 +43,10 @@ __device__ __forceinline__ float activate(float s) {
 template <int ACT>
 __device__ __forceinline__ float activate_slope(float s) {
   if (ACT == OT_ACT_TANH) {
-    const float a = tanh_dev(s);
-    return 1.f - a * a;
+    // 1 - tanh^2 = 4e / (1 + e)^2 with e = exp(-2|s|): no cancellation near |tanh| = 1
+    const float e = __builtin_amdgcn_exp2f(__builtin_fabsf(s) * -2.88539004325866699219f);
+    const float r = __builtin_amdgcn_rcpf(1.f + e);
+    return 4.f * e * (r * r);
   }
   return 1.f;
 }
