@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "ot_device.hip.h"
 #include "ot_transducer.h"
 
@@ -328,7 +330,7 @@ template <bool BETA, bool OSF, bool MULTI>
 __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int T, int U,
                                               int64_t row0, float *__restrict__ out,
                                               float *__restrict__ score,
-                                              float (*s_ring)[kRing + 1]) {
+                                              float (*s_ring)[kRing + kChunk]) {
   const int u = threadIdx.x;
   const int lane = u & (kWave - 1), wave = u / kWave;
   const int U1 = U + 1;
@@ -365,11 +367,16 @@ __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int 
   // wave whose edge lane feeds this wave, if any
   const int src_wave = BETA ? wave + 1 : wave - 1;
   const bool has_src = MULTI && src_wave >= 0 && src_wave <= wlast;
+  const int src_ok = has_src ? src_wave : wave;  // a ring that exists, for the unconditional read
   const int edge_lane = BETA ? 0 : kWave - 1;
-  // where this lane's per-step ring write goes: the edge lane publishes, every
-  // other lane hits a dummy slot behind the ring
+  // where this lane's per-step ring writes go: the edge lane publishes, every
+  // other lane hits kChunk dummy slots behind the ring
   float *const ring_dst = &s_ring[wave][(lane == edge_lane) ? 0 : kRing];
   const int ring_mask = (lane == edge_lane) ? (kRing - 1) : 0;
+  // lane that holds the edge value of step i of a chunk when the chunk starts: the
+  // register is rotated by one lane per step towards the lane that consumes it
+  // (lane 0 of an alpha wave, lane 63 of a beta wave)
+  const int ering_step = BETA ? (kWave - 1 - lane) : lane;
 
   // alpha: own = alpha(t-1,u)+blank(t-1,u), nb = alpha(t,u)+sym(t,u) handed to u+1
   // beta : own = nb = beta of the cell computed in the previous step
@@ -392,19 +399,21 @@ __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int 
     // the kChunk edge values of this chunk were all written before the last
     // barrier: fetch them with one LDS read, one lane each
     float ering = OT_NEG_INF;
+    float *ring_wr = nullptr;
     if (MULTI) {
-      const int s = n - 1 - kLag + lane;
-      if (has_src && lane < kChunk && s >= 0) ering = s_ring[src_wave][s & (kRing - 1)];
+      // read without a branch (any slot of a valid wave's ring is readable), then select:
+      // a branch here splits the loop body and costs register copies of the prefetch ring
+      const int s = n - 1 - kLag + ering_step;
+      const float v = s_ring[src_ok][s & (kRing - 1)];
+      ering = (has_src && ering_step < kChunk && s >= 0) ? v : OT_NEG_INF;
+      ring_wr = ring_dst + (n & ring_mask);  // n is a multiple of kChunk: no wrap inside a chunk
     }
 #pragma unroll
     for (int i = 0; i < kChunk; ++i) {
       const f32x2 l = q[i];
-      q[i] = fetch(off_lp);
-      float edge = OT_NEG_INF;
-      if (MULTI)
-        edge = __builtin_bit_cast(
-            float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ering), i));
-      const float in = BETA ? wave_shift_down(nb, edge) : wave_shift_up(nb, edge);
+      // the lane without a source lane keeps the fill value: the edge of this step
+      const float in = BETA ? wave_shift_down(nb, ering) : wave_shift_up(nb, ering);
+      if (MULTI) ering = BETA ? dpp_mov<kDppWaveShr1>(ering) : dpp_mov<kDppWaveShl1>(ering);
       float a = BETA ? log_add(own + l.x, in + l.y) : log_add(own, in);
       if (OSF) a = ((unsigned)(t - u) < band) ? a : OT_NEG_INF;
       __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, a), out_buf, off_out, 0, 0);
@@ -414,7 +423,10 @@ __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int 
         own = a + l.x;
         nb = a + l.y;
       }
-      if (MULTI) ring_dst[(n + i) & ring_mask] = nb;
+      if (MULTI) ring_wr[i] = nb;
+      // refill the slot only now that l is dead: issued earlier, the load needs a second
+      // register pair and the loop ends in copies that wait for the loads in flight
+      q[i] = fetch(off_lp);
       if (OSF) t += dt;
       off_out += d_out;
       off_lp += d_lp;
@@ -435,13 +447,164 @@ __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int 
   }
 }
 
+// ---------------------------------------------------------------------------
+// Standard lattice with three or more waves per workgroup.
+//
+// On the anti-diagonal wavefront the 64 lanes of a wave touch 64 different rows of
+// lp and of alpha/beta in every step: 64 cache lines per load and per store
+// instruction, and from three waves on the CU's address unit, not the recursion,
+// sets the pace.  Here the lanes of a group of G consecutive columns access the
+// SAME row in one instruction, G*8 (lp) or G*4 (alpha/beta) contiguous bytes:
+//   - lp: every lane loads its own column's value of a row that lies kk + 18 steps
+//     ahead of it, kk = its distance from the group's leading lane (0..G-1); the
+//     value waits in a wave-private LDS ring of G rows until the lane gets there;
+//   - alpha/beta: every lane parks its result in a second LDS ring and stores the
+//     one it computed G-1-kk steps ago, which lies in the row the group's trailing
+//     lane has just finished.
+// A lane only ever reads LDS slots it wrote itself, in program order, so the
+// staging needs no synchronisation; LDS reads are issued two steps before use.
+// The recursion, the cross-wave hand-over and the barrier per kChunk steps are
+// those of lattice_sweep.  Two compute-free chunks fill the rings first.
+// ---------------------------------------------------------------------------
+constexpr int kStageLead = kChunk + 2;   // steps between a load and its use, for kk = 0
+constexpr int kStageWarmup = 2 * kChunk; // compute-free steps in front
+
+template <bool BETA, int G>
+__device__ __forceinline__ void lattice_sweep_staged(const float *__restrict__ lp, int T, int U,
+                                                     int64_t row0, float *__restrict__ out,
+                                                     float *__restrict__ score,
+                                                     float (*s_ring)[kRing + kChunk],
+                                                     float *s_stage) {
+  static_assert(G >= 2 && G <= kChunk && (G & (G - 1)) == 0, "group size");
+  const int u = threadIdx.x;
+  const int lane = u & (kWave - 1), wave = u / kWave;
+  const int nwaves = blockDim.x / kWave;
+  const int U1 = U + 1;
+  const int wlast = U / kWave;
+  const int nsteps = T + U + wlast * kLag;
+  const bool column = u < U1;
+  const int delay = BETA ? (U - u) + (wlast - wave) * kLag : u + wave * kLag;
+  const int kk = BETA ? (G - 1 - (lane & (G - 1))) : (lane & (G - 1));
+  const int jj = (G - 1) - kk;
+
+  const unsigned cells = (unsigned)T * (unsigned)U1;
+  const __amdgpu_buffer_rsrc_t lp_buf = make_buffer(lp + 2 * row0, cells * 8u);
+  const __amdgpu_buffer_rsrc_t out_buf = make_buffer(out + row0, cells * 4u);
+  const unsigned oob = column ? 0u : 0x80000000u;
+  const int dcell = BETA ? -U1 : U1;
+  const int t0 = BETA ? (T - 1 + delay) : -delay;  // lattice row at step 0
+  const int cell0 = t0 * U1 + u;
+  const unsigned d_out = (unsigned)dcell * 4u, d_lp = (unsigned)dcell * 8u;
+  // step n loads the lp cell of step n + kChunk + kStageLead + kk - kChunk ... in full:
+  // issued at step n, in a register until step n + kChunk, in LDS until step n + kChunk + kk + 2
+  unsigned off_lp = (unsigned)(cell0 + (kStageLead + kk - kStageWarmup) * dcell) * 8u + oob;
+  // step n stores the cell of step n - 2 - jj
+  unsigned off_st = (unsigned)(cell0 - (2 + jj) * dcell) * 4u + oob;
+
+  auto fetch = [&](unsigned byte_off) -> f32x2 {
+    return __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(lp_buf, byte_off, 0, 0));
+  };
+
+  f32x2 *const lp_ring = reinterpret_cast<f32x2 *>(s_stage) + wave * (G * kWave) + lane;
+  float *const out_ring = s_stage + nwaves * (2 * G * kWave) + wave * (G * kWave) + lane;
+
+  const int src_wave = BETA ? wave + 1 : wave - 1;
+  const bool has_src = src_wave >= 0 && src_wave <= wlast;
+  const int src_ok = has_src ? src_wave : wave;
+  const int edge_lane = BETA ? 0 : kWave - 1;
+  float *const ring_dst = &s_ring[wave][(lane == edge_lane) ? 0 : kRing];
+  const int ring_mask = (lane == edge_lane) ? (kRing - 1) : 0;
+  const int ering_step = BETA ? (kWave - 1 - lane) : lane;
+
+  float own = (column && u == (BETA ? U : 0)) ? 0.f : OT_NEG_INF;
+  float nb = OT_NEG_INF;
+
+  f32x2 q[kChunk];
+#pragma unroll
+  for (int i = 0; i < kChunk; ++i)
+    q[i] = fetch((unsigned)(cell0 + (i - kChunk + kStageLead + kk - kStageWarmup) * dcell) * 8u + oob);
+  f32x2 lpipe[2] = {{0.f, 0.f}, {0.f, 0.f}};
+  float spipe[2] = {0.f, 0.f};
+
+  // kChunk steps starting at step n (a multiple of kChunk); LIVE = false only stages lp
+  auto chunk = [&](auto live_tag, int n) {
+    constexpr bool LIVE = decltype(live_tag)::value;
+    float ering = OT_NEG_INF;
+    float *ring_wr = nullptr;
+    if (LIVE) {
+      const int s = n - 1 - kLag + ering_step;
+      const float v = s_ring[src_ok][s & (kRing - 1)];
+      ering = (has_src && ering_step < kChunk && s >= 0) ? v : OT_NEG_INF;
+      ring_wr = ring_dst + (n & ring_mask);
+    }
+#pragma unroll
+    for (int i = 0; i < kChunk; ++i) {
+      // lp: register -> LDS slot of the step that uses it; LDS -> register for step i + 2
+      lp_ring[((i + kk + 2) & (G - 1)) * kWave] = q[i];
+      q[i] = fetch(off_lp);
+      off_lp += d_lp;
+      const f32x2 l = lpipe[i & 1];
+      lpipe[i & 1] = lp_ring[((i + 2) & (G - 1)) * kWave];
+      if (LIVE) {
+        const float in = BETA ? wave_shift_down(nb, ering) : wave_shift_up(nb, ering);
+        ering = BETA ? dpp_mov<kDppWaveShr1>(ering) : dpp_mov<kDppWaveShl1>(ering);
+        const float a = BETA ? log_add(own + l.x, in + l.y) : log_add(own, in);
+        out_ring[(i & (G - 1)) * kWave] = a;
+        const float st = spipe[i & 1];
+        spipe[i & 1] = out_ring[((i + kk + 1) & (G - 1)) * kWave];  // slot of step i - jj
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, st), out_buf, off_st, 0, 0);
+        off_st += d_out;
+        if (BETA) {
+          own = nb = a;
+        } else {
+          own = a + l.x;
+          nb = a + l.y;
+        }
+        ring_wr[i] = nb;
+      }
+    }
+    if (LIVE) lds_barrier();
+  };
+
+  for (int n = -kStageWarmup; n < 0; n += kChunk) chunk(std::false_type{}, n);
+  // the last cell's store trails its computation by up to G + 1 steps
+  for (int n = 0; n < nsteps + G + 1; n += kChunk) chunk(std::true_type{}, n);
+
+  if (column && u == (BETA ? 0 : U)) {
+    __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have completed
+    if (BETA) {
+      *score = out[row0];
+    } else {
+      const int64_t last = row0 + (int64_t)cells - 1;
+      *score = out[last] + lp[2 * last];
+    }
+  }
+}
+
+template <int G, int THREADS>
+__global__ __launch_bounds__(THREADS) void alpha_beta_staged_kernel(
+    const float *__restrict__ lp, const int32_t *__restrict__ logit_lengths,
+    const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
+    int utt_begin, float *__restrict__ alpha, float *__restrict__ beta,
+    float *__restrict__ scores_alpha, float *__restrict__ scores_beta) {
+  __shared__ float s_ring[THREADS / kWave][kRing + kChunk];
+  extern __shared__ __attribute__((aligned(16))) float s_stage[];
+  const int b = utt_begin + blockIdx.x;
+  const int T = logit_lengths[b], U = target_lengths[b];
+  const int64_t row0 = row_splits[b];
+  if (blockIdx.y == 0)
+    lattice_sweep_staged<false, G>(lp, T, U, row0, alpha, scores_alpha + b, s_ring, s_stage);
+  else
+    lattice_sweep_staged<true, G>(lp, T, U, row0, beta, scores_beta + b, s_ring, s_stage);
+}
+
 template <bool OSF, bool MULTI>
 __global__ __launch_bounds__(OT_MAX_U1) void alpha_beta_kernel(
     const float *__restrict__ lp, const int32_t *__restrict__ logit_lengths,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
     int utt_begin, float *__restrict__ alpha, float *__restrict__ beta,
     float *__restrict__ scores_alpha, float *__restrict__ scores_beta) {
-  __shared__ float s_ring[MULTI ? kMaxDpWaves : 1][kRing + 1];
+  __shared__ float s_ring[MULTI ? kMaxDpWaves : 1][kRing + kChunk];
   const int b = utt_begin + blockIdx.x;
   const int T = logit_lengths[b], U = target_lengths[b];
   const int64_t row0 = row_splits[b];
@@ -778,6 +941,21 @@ int ot_alpha_beta_range(const float *lp, const int32_t *logit_lengths,
   const int threads = ((max_u1 + kWave - 1) / kWave) * kWave;
   const dim3 grid((unsigned)(utt_end - utt_begin), 2), block((unsigned)threads);
   const bool multi = threads > kWave;
+  const int nwaves = threads / kWave;
+  if (!one_sym_per_frame && nwaves >= 3) {
+    // staging rings: (8 + 4) bytes per lane and group row
+    const int G = nwaves <= 4 ? 16 : nwaves <= 9 ? 8 : 4;
+    const size_t lds = (size_t)nwaves * G * kWave * 12;
+#define OT_LAUNCH_DPS(G_, THREADS_)                                                             \
+  hipLaunchKernelGGL((alpha_beta_staged_kernel<G_, THREADS_>), grid, block, lds, s, lp,         \
+                     logit_lengths, target_lengths, row_splits, utt_begin, alpha, beta,         \
+                     scores_alpha, scores_beta)
+    if (G == 16) OT_LAUNCH_DPS(16, 256);
+    else if (G == 8) OT_LAUNCH_DPS(8, 576);
+    else OT_LAUNCH_DPS(4, 1024);
+#undef OT_LAUNCH_DPS
+    return launch_status();
+  }
 #define OT_LAUNCH_DP(OSF_, MULTI_)                                                              \
   hipLaunchKernelGGL((alpha_beta_kernel<OSF_, MULTI_>), grid, block, 0, s, lp, logit_lengths,   \
                      target_lengths, row_splits, utt_begin, alpha, beta, scores_alpha, scores_beta)

@@ -119,6 +119,44 @@ def test_lattice_kernel_given_oracle_log_probs(case, device):
     assert (a2.cpu().numpy() == a).all() and (b2.cpu().numpy() == b).all()
 
 
+WIDE = [  # (T, U) per utterance: 3..16 waves per workgroup, mixed with short targets
+    ("three_waves", [(50, 130), (9, 191), (20, 5)]),
+    ("four_waves", [(300, 200), (7, 255), (64, 64), (1, 250)]),
+    ("five_waves", [(40, 300), (3, 319), (100, 0)]),
+    ("nine_waves", [(33, 575), (100, 577), (5, 70)]),
+    ("ten_waves", [(25, 600), (1, 639), (80, 129)]),
+    ("sixteen_waves", [(40, 1023), (3, 700), (17, 1000), (30, 63)]),
+]
+
+
+@pytest.mark.parametrize("osf", [False, True])
+@pytest.mark.parametrize("name,shapes", WIDE, ids=[w[0] for w in WIDE])
+def test_lattice_kernel_with_many_waves(name, shapes, osf, device):
+    rng = np.random.default_rng(len(name))
+    T = np.array([s[0] for s in shapes], np.int32)
+    U = np.array([s[1] for s in shapes], np.int32)
+    if osf:
+        T = np.maximum(T, U + 1 + rng.integers(0, 40, size=len(T))).astype(np.int32)
+    rows = int((T.astype(np.int64) * (U + 1)).sum())
+    # log-probabilities of a plausible size; lp[., 1] at u == U is never read
+    lp = (-rng.random((rows, 2)) * 6 - 0.05).astype(np.float32)
+    fn_a = oracle.alpha if not osf else (lambda *a: oracle.alpha(*a, one_sym_per_frame=True))
+    fn_b = oracle.beta if not osf else (lambda *a: oracle.beta(*a, one_sym_per_frame=True))
+    wa, sa_w = fn_a(lp, T, U)
+    wb, sb_w = fn_b(lp, T, U)
+    dT, dU = _dev(T, device), _dev(U, device)
+    splits, _ = cabi.row_splits(dT, dU, torch.zeros((len(T), 0), dtype=torch.int32, device=device))
+    a, b, sa, sb = cabi.alpha_beta(_dev(lp, device), dT, dU, splits, int(U.max()) + 1, osf)
+    a, b, sa, sb = (t.cpu().numpy() for t in (a, b, sa, sb))
+    for got, want in ((a, wa), (b, wb)):
+        m = ~np.isnan(want)
+        assert np.allclose(got[m], want[m], rtol=RTOL, atol=ATOL), np.abs(got[m] - want[m]).max()
+        assert np.isneginf(got[~m]).all()
+    assert np.allclose(sa, sa_w, rtol=RTOL, atol=ATOL) and np.allclose(sb, sb_w, rtol=RTOL, atol=ATOL)
+    a2, b2, _, _ = cabi.alpha_beta(_dev(lp, device), dT, dU, splits, int(U.max()) + 1, osf)
+    assert (a2.cpu().numpy() == a).all() and (b2.cpu().numpy() == b).all()
+
+
 @pytest.mark.parametrize("fls", [False, True])
 @pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
 def test_gradient_kernels_given_oracle_lattice(case, fls, device):
