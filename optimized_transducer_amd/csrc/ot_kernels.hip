@@ -157,8 +157,6 @@ __global__ __launch_bounds__(kBlock) void lse_gather_kernel(
   // this launch covers rows [row_begin, rows)
   const int64_t row_first = row_begin + (int64_t)blockIdx.x * rows_per_block;
   const int64_t row_end = min(rows, row_first + rows_per_block);
-  bu.load(row_splits, N, row_first, row_end - 1);
-  const int64_t lattice_rows = row_splits[N];
 
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sub = lane % L, g = lane / L;
@@ -180,6 +178,10 @@ __global__ __launch_bounds__(kBlock) void lse_gather_kernel(
 
   int64_t base = row_first + (int64_t)wave * G;
   if (kStaged && whole_row && base < row_end) issue_span(base);
+  // the utterance table is only needed for the gather at the end of a pass: its
+  // searches run while the first span is in flight
+  bu.load(row_splits, N, row_first, row_end - 1);
+  const int64_t lattice_rows = row_splits[N];
 
   for (; base < row_end; base += kWavesPerBlock * G) {
     const int64_t row = base + g;
