@@ -54,11 +54,12 @@ __device__ __forceinline__ float activate_slope(float s) {
 // ---------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------
-// One workgroup = utterance b, kPackFrames frames, all positions u,
+// One workgroup = utterance b, kPackFrames frames, kPackPositions positions u,
 // up to 256 column units.  A thread keeps its columns of the frames' encoder rows
 // in registers and walks u: one decoder load serves kPackFrames output rows, no
 // index array is read, and every store instruction of a wave writes a contiguous
 // piece of one output row.
+constexpr int kPackPositions = 16;  // positions u per workgroup: fastest of 8, 16, 32, 64, all
 constexpr int kPackFrames = 2;  // fastest of 1, 2, 4, 8 on MI355X
 
 template <int VEC, int ACT>
@@ -76,8 +77,11 @@ __global__ __launch_bounds__(kBlock) void joiner_pack_kernel(
   const int cpb = min(nvec, kBlock);  // column units per workgroup
   const int phases = kBlock / cpb;    // positions u in flight per workgroup
   const int phase = threadIdx.x / cpb;
-  const int unit = blockIdx.x * cpb + (threadIdx.x - phase * cpb);
-  if (phase >= phases || unit >= nvec) return;
+  const int nslabs = (nvec + cpb - 1) / cpb;
+  const int uc = blockIdx.x / nslabs, slab = blockIdx.x - uc * nslabs;
+  const int u_begin = uc * kPackPositions, u_end = min(U1, u_begin + kPackPositions);
+  const int unit = slab * cpb + (threadIdx.x - phase * cpb);
+  if (phase >= phases || unit >= nvec || u_begin >= U1) return;
   const int col = unit * VEC;
   const int nt = min(kPackFrames, T - t0);
   Vec<VEC> e[kPackFrames];
@@ -91,10 +95,10 @@ __global__ __launch_bounds__(kBlock) void joiner_pack_kernel(
   const float *dp = dec + ((int64_t)b * u_stride * D + col);
   const int64_t frame_stride = (int64_t)U1 * D;
   Vec<VEC> d;
-  if (phase < U1) d.load_cached(dp + (int64_t)phase * D);
-  for (int u = phase; u < U1; u += phases) {
+  if (u_begin + phase < u_end) d.load_cached(dp + (int64_t)(u_begin + phase) * D);
+  for (int u = u_begin + phase; u < u_end; u += phases) {
     Vec<VEC> dn = d;
-    if (u + phases < U1) dn.load_cached(dp + (int64_t)(u + phases) * D);
+    if (u + phases < u_end) dn.load_cached(dp + (int64_t)(u + phases) * D);
 #pragma unroll
     for (int i = 0; i < kPackFrames; ++i) {
       if (i < nt) {
@@ -289,7 +293,7 @@ int ot_joiner_pack(const float *enc, const float *dec, const int32_t *logit_leng
   const int vec = (D % 4 == 0 && aligned16(enc) && aligned16(dec) && aligned16(out)) ? 4 : 1;
   const int nvec = D / vec;
   const int cpb = nvec < kBlock ? nvec : kBlock;
-  const dim3 grid((unsigned)((nvec + cpb - 1) / cpb),
+  const dim3 grid((unsigned)(((nvec + cpb - 1) / cpb) * ((u_stride + kPackPositions - 1) / kPackPositions)),
                   (unsigned)((t_stride + kPackFrames - 1) / kPackFrames), (unsigned)N);
 #define OT_LAUNCH_PACKT(VEC_, ACT_)                                                             \
   hipLaunchKernelGGL((joiner_pack_kernel<VEC_, ACT_>), grid, dim3(kBlock), 0, s, enc, dec, \
