@@ -197,6 +197,13 @@ size_t ot_gradient_scratch_bytes(int64_t rows);
 int ot_scale_by_device_scalar(float *x, int64_t n, const float *factor,
                               void *stream);
 
+/* *loss = -scale * sum_b scores[b]: the reduction of the per-utterance
+ * log-likelihoods to the loss (transducer_loss.py:145-147: loss = -1 * scores,
+ * then .sum() or .mean(); pass scale = 1 or 1/N).  One launch, fixed summation
+ * order. */
+int ot_negative_sum(const float *scores, int32_t N, float scale, float *loss,
+                    void *stream);
+
 /* Bytes of device scratch ot_transducer_loss needs for N utterances and
  * `rows` packed rows. */
 size_t ot_workspace_bytes(int32_t N, int64_t rows);

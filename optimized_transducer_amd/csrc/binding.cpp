@@ -422,6 +422,21 @@ torch::Tensor apply_deferred_gradient(torch::Tensor &logits, const torch::Tensor
   return gradient;
 }
 
+// 0-dim loss = -scale * scores.sum() in one launch (replaces `-1 * scores` followed
+// by .sum() / .mean(), transducer_loss.py:145-147).
+torch::Tensor negative_sum(const torch::Tensor &scores, double scale) {
+  TORCH_CHECK(scores.is_cuda() && scores.scalar_type() == torch::kFloat && scores.dim() == 1 &&
+                  scores.is_contiguous() && scores.numel() > 0 && scores.numel() <= INT32_MAX,
+              "negative_sum: scores must be a non-empty contiguous 1-D float32 HIP tensor");
+  c10::hip::HIPGuardMasqueradingAsCUDA device_guard(scores.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+  torch::Tensor loss = torch::empty({}, scores.options());
+  ScopedTimer timer("negative_sum", stream);
+  OT_CHECK(ot_negative_sum(scores.data_ptr<float>(), (int32_t)scores.numel(), (float)scale,
+                           loss.data_ptr<float>(), stream));
+  return loss;
+}
+
 // x *= loss_grad with loss_grad read on the device (no host synchronisation);
 // the kernel returns immediately when loss_grad == 1.
 void scale_by_device_scalar_(torch::Tensor &x, const torch::Tensor &factor) {
@@ -581,6 +596,8 @@ PYBIND11_MODULE(_optimized_transducer, m) {
         py::arg("loss_grad"),
         "The (rows, V) gradient pass for the coefficients of compute_transducer_loss_deferred, "
         "times grad_scale and the device scalar loss_grad.");
+  m.def("negative_sum", &negative_sum, py::arg("scores"), py::arg("scale"),
+        "0-dim tensor -scale * scores.sum(), one launch.");
   m.def("scale_by_device_scalar_", &scale_by_device_scalar_, py::arg("x"), py::arg("factor"));
   m.def("joiner_pack", &joiner_pack, py::arg("encoder_out"), py::arg("decoder_out"),
         py::arg("logit_lengths"), py::arg("target_lengths"), py::arg("activation"),

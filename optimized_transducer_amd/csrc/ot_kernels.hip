@@ -10,6 +10,7 @@
 //   row_coeff_kernel      per-row part of the gradients  kernels.cu:522-779
 //   grad_flat_kernel      (rows, V) pass of the gradients kernels.cu:522-779
 //   scale_kernel          grad *= loss_grad              transducer_loss.py:162
+//   negative_sum_kernel   loss = -sum or -mean of scores transducer_loss.py:145-147
 //
 // The two kernels that move (rows, V) data are HBM-bound streaming kernels: a
 // group of L lanes owns one row, every lane keeps K 128-bit vectors of the row
@@ -805,6 +806,24 @@ __global__ __launch_bounds__(kBlock) void scale_kernel(float *__restrict__ x, in
   }
 }
 
+// loss = -scale * sum(scores): one workgroup, fixed summation order
+__global__ __launch_bounds__(kBlock) void negative_sum_kernel(const float *__restrict__ scores,
+                                                              int n, float scale,
+                                                              float *__restrict__ loss) {
+  __shared__ float s_part[kWavesPerBlock];
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < n; i += kBlock) acc += scores[i];
+  acc = group_allreduce<kWave>(acc, SumOp());
+  if ((threadIdx.x & (kWave - 1)) == 0) s_part[threadIdx.x / kWave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) t += s_part[w];
+    *loss = -(t * scale);
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void copy_kernel(const float4 *__restrict__ src,
                                                       float4 *__restrict__ dst, int64_t n4) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -1152,6 +1171,13 @@ int ot_transducer_loss(const float *logits, const int32_t *targets, const int32_
                      row_splits, N, targets_cols, rows, V, blank, from_log_softmax,
                      one_sym_per_frame, grad_scale, row_scratch, grad, stream);
   return rc;
+}
+
+int ot_negative_sum(const float *scores, int32_t N, float scale, float *loss, void *stream) {
+  if (!scores || !loss || N <= 0) return OT_E_BAD_ARG;
+  hipLaunchKernelGGL(negative_sum_kernel, dim3(1), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                     scores, N, scale, loss);
+  return launch_status();
 }
 
 int ot_copy_floats(const float *src, float *dst, int64_t n, void *stream) {

@@ -5,6 +5,8 @@ Differences from the reference that do not change results:
 
 * the ``grad /= N`` pass of ``reduction="mean"`` (transducer_loss.py:150) is
   folded into the gradient kernel as a multiplication by ``1/N``;
+* ``-1 * scores`` and the ``.sum()`` / ``.mean()`` that follows
+  (transducer_loss.py:145-147) are one launch with a fixed summation order;
 * ``backward`` multiplies by ``loss_grad`` with a kernel that reads the factor
   on the device and does nothing when it equals 1 (transducer_loss.py:162 always
   makes a full pass);
@@ -69,8 +71,7 @@ class TransducerLossFunction(torch.autograd.Function):
                 # backward is then reported instead of giving a wrong gradient
                 ctx.save_for_backward(logits)
                 ctx.deferred = (coefficients, from_log_softmax, grad_scale)
-            loss = -1 * scores
-            return loss.mean() if reduction == "mean" else loss.sum()
+            return _optimized_transducer.negative_sum(scores, grad_scale)
 
         scores, grad = _optimized_transducer.compute_transducer_loss_scaled(
             logits=logits,
@@ -83,11 +84,8 @@ class TransducerLossFunction(torch.autograd.Function):
             grad_scale=grad_scale,
         )
 
-        loss = -1 * scores
-        if reduction == "mean":
-            loss = loss.mean()
-        elif reduction == "sum":
-            loss = loss.sum()
+        # loss = -1 * scores, then .mean() or .sum() (reference transducer_loss.py:145-147)
+        loss = _optimized_transducer.negative_sum(scores, grad_scale)
 
         ctx.grad = grad
         return loss

@@ -179,3 +179,10 @@ def joiner_unpack_grad(grad_out, enc, dec, T, U, splits, activation):
                                   ctypes.c_int32(activation), ptr(ws), ctypes.c_size_t(nbytes),
                                   ptr(ge), ptr(gd), stream()))
     return ge, gd
+
+
+def negative_sum(scores, scale):
+    loss = torch.full((1,), float("nan"), dtype=torch.float32, device=scores.device)
+    check(lib().ot_negative_sum(ptr(scores), ctypes.c_int32(scores.numel()), ctypes.c_float(scale),
+                                ptr(loss), stream()))
+    return loss

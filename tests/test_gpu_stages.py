@@ -234,6 +234,21 @@ def test_scale_by_device_scalar(device):
     assert torch.equal(y, ref[1:] * 3.0 * 3.0)
 
 
+def test_negative_sum(device):
+    # loss = -scale * sum(scores) (transducer_loss.py:145-147), fixed order: same bits twice
+    rng = np.random.default_rng(8)
+    for n in (1, 3, 64, 257, 5000):
+        x = (-rng.random(n) * 3000).astype(np.float32)
+        d = _dev(x, device)
+        for scale in (1.0, 1.0 / n):
+            got = cabi.negative_sum(d, scale).item()
+            want = -float(np.float32(scale)) * x.astype(np.float64).sum()
+            assert abs(got - want) <= 1e-6 * abs(want), (n, scale, got, want)
+            assert cabi.negative_sum(d, scale).item() == got
+    inf = _dev(np.array([-1.0, -np.inf], np.float32), device)
+    assert cabi.negative_sum(inf, 1.0).item() == np.inf
+
+
 def test_copy_floats(device):
     a = torch.randn(1 << 20, device=device)
     b = torch.zeros_like(a)
