@@ -15,6 +15,16 @@ except ImportError as e:  # pragma: no cover - exercised only on an unbuilt tree
         "Run `python -m optimized_transducer_amd.build` in the repository root." % (e,)
     ) from e
 
+import torch as _torch
+
+# same guard as the reference package (optimized_transducer/__init__.py:5-9)
+_built = getattr(_optimized_transducer, "built_with_torch", _torch.__version__)
+if _torch.__version__.split("+")[0] != _built.split("+")[0]:
+    raise ImportError(
+        f"optimized_transducer_amd was built using PyTorch {_built}\n"
+        f"But you are using PyTorch {_torch.__version__} to run it"
+    )
+
 from .transducer_loss import TransducerLoss, TransducerLossFunction, transducer_loss  # noqa: E402,F401
 from .joiner import PackJoinerFunction, pack_joiner  # noqa: E402,F401
 

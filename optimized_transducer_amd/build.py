@@ -49,6 +49,7 @@ def build_extension():
         "g++", "-O2", "-std=c++17", "-fPIC", "-shared",
         "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
         "-DTORCH_EXTENSION_NAME=_optimized_transducer",
+        '-DOT_BUILT_WITH_TORCH="%s"' % torch.__version__,
         "-D_GLIBCXX_USE_CXX11_ABI=%d" % abi,
         "-I", INCLUDE,
         "-I", os.path.join(tdir, "include"),

@@ -578,6 +578,11 @@ std::pair<torch::Tensor, torch::Tensor> joiner_unpack_grad(
 
 PYBIND11_MODULE(_optimized_transducer, m) {
   m.doc() = "MI355X-native transducer loss (drop-in for optimized_transducer's extension module)";
+#ifdef OT_BUILT_WITH_TORCH
+  // the reference records the same fact in a generated torch_version.py
+  // (optimized_transducer/python/optimized_transducer/__init__.py:3-9)
+  m.attr("built_with_torch") = OT_BUILT_WITH_TORCH;
+#endif
   m.def("compute_transducer_loss", &compute_transducer_loss, py::arg("logits"),
         py::arg("targets"), py::arg("logit_lengths"), py::arg("target_lengths"),
         py::arg("blank"), py::arg("from_log_softmax"), py::arg("one_sym_per_frame"));
