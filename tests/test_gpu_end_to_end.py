@@ -195,6 +195,72 @@ def test_reference_test_shapes_modified_logits_vs_logsoftmax(device):
     assert np.allclose(a.grad.cpu().numpy(), want, atol=1e-4)
 
 
+def _cat_of_leaves(x, T, U, device):
+    # the reference tests build logits as cat([leaf0, leaf1]) and read the leaves' grads
+    sizes = (T.astype(np.int64) * (U + 1)).tolist()
+    leaves = [t.clone().requires_grad_(True) for t in torch.split(_dev(x, device), sizes)]
+    return leaves, torch.cat(leaves)
+
+
+@pytest.mark.parametrize("reduction", ["mean", "sum"])
+def test_reference_test_shapes_small(reduction, device):
+    # test_cuda.py:15-70 (T=3/4, U+1=3/3, V=3; device result == CPU result) and
+    # test_log_softmax.py:25-86 (T=8/5, U+1=4/5, V=3; logits path == log-softmax path,
+    # atol 1e-3), targets = randint(1, V-1) = all ones, rand logits
+    import optimized_transducer_amd as ot
+    rng = np.random.default_rng(20211227)
+    for Ts, U1s in (((3, 4), (3, 3)), ((8, 5), (4, 5))):
+        T = np.array(Ts, np.int32)
+        U = np.array(U1s, np.int32) - 1
+        V = 3
+        tg = np.ones((2, int(U.max())), np.int32)
+        x = rng.random((int((T * (U + 1)).sum()), V), dtype=np.float32)
+        dtg, dT, dU = _dev(tg, device), _dev(T, device), _dev(U, device)
+        leaves, logits = _cat_of_leaves(x, T, U, device)
+        loss = ot.transducer_loss(logits=logits, targets=dtg, logit_lengths=dT, target_lengths=dU,
+                                  blank=0, from_log_softmax=False, reduction=reduction)
+        loss.backward()
+        leaves2, _ = _cat_of_leaves(x, T, U, device)
+        loss2 = ot.transducer_loss(logits=torch.cat([l.log_softmax(-1) for l in leaves2]),
+                                   targets=dtg, logit_lengths=dT, target_lengths=dU, blank=0,
+                                   from_log_softmax=True, reduction=reduction)
+        loss2.backward()
+        want_loss, want = oracle.transducer_loss(x.copy(), tg, T, U, 0, False, False, reduction)
+        assert torch.allclose(loss, loss2, atol=1e-3) and np.allclose(loss.item(), want_loss, atol=1e-6,
+                                                                       rtol=1e-6)
+        got = torch.cat([l.grad for l in leaves]).cpu().numpy()
+        got2 = torch.cat([l.grad for l in leaves2]).cpu().numpy()
+        assert np.allclose(got, got2, atol=1e-3)
+        assert np.allclose(got, want, rtol=RTOL, atol=ATOL) and np.allclose(got2, want, rtol=1e-4,
+                                                                             atol=ATOL)
+
+
+def test_reference_test_shapes_large(device):
+    # test_compute_transducer_loss.py:28-105: T in [100,1000) / [500,2000), U+1 in [100,300) /
+    # [20,500), V in [5,100), rand logits, loss * 3 before backward, compared there with
+    # torchaudio at atol 1e-3 (loss, first utterance) and 1e-2 (second); here with the CPU oracle
+    import optimized_transducer_amd as ot
+    rng = np.random.default_rng(20211230)
+    T = np.array([rng.integers(100, 1000), rng.integers(500, 2000)], np.int32)
+    U = np.array([rng.integers(100, 300), rng.integers(20, 500)], np.int32) - 1
+    V = int(rng.integers(5, 100))
+    tg = rng.integers(1, V - 1, size=(2, int(U.max()))).astype(np.int32)
+    x = rng.random((int((T.astype(np.int64) * (U + 1)).sum()), V), dtype=np.float32)
+    leaves, logits = _cat_of_leaves(x, T, U, device)
+    loss = ot.transducer_loss(logits=logits, targets=_dev(tg, device), logit_lengths=_dev(T, device),
+                              target_lengths=_dev(U, device), blank=0, from_log_softmax=False,
+                              reduction="mean")
+    (loss * 3).backward()
+    want_loss, want = oracle.transducer_loss(x.copy(), tg, T, U, 0, False, False, "mean",
+                                             loss_grad=3.0)
+    assert abs(loss.item() - want_loss) <= 1e-3
+    got = torch.cat([l.grad for l in leaves]).cpu().numpy()
+    assert np.abs(got - want).max() <= 1e-3
+    s, _ = oracle.compute_transducer_loss(x.copy(), tg, T, U, 0, False, False)
+    tol = 1.5 * helpers.lattice_noise_tolerance(want / 1.5, helpers.per_row(s, T, U))
+    assert (np.abs(got - want) <= tol).all(), np.abs(got - want).max()
+
+
 def test_two_stream_schedule_gives_the_same_bits(device):
     # opt-in schedule: lattice kernel of one half of the batch on a second stream
     import optimized_transducer_amd as ot
