@@ -400,6 +400,9 @@ FULL = [
     ("largevocab", lambda: workloads.large_vocab()),
     ("ragged", lambda: workloads.ragged()),
     ("ragged_modified", lambda: workloads.ragged(one_sym_per_frame=True)),
+    # more than 2^31 logits: element offsets need 64 bits (the reference's CUDA kernels
+    # index with int there, kernels.cu:49)
+    ("beyond_int32", lambda: workloads.beyond_int32()),
 ]
 
 
@@ -420,11 +423,18 @@ def test_full_size_workloads(name, make, device):
     sizes = T.astype(np.int64) * (U + 1)
     pick = sorted(set([int(np.argmax(T + U)), 0, len(T) - 1]
                       + [int(i) for i in np.where((T == 1) | (U == 0))[0][:4]]))
+    huge = x.numel() > 2 ** 31
+    if huge:  # the first and the last utterance only: the last one straddles element 2^31
+        pick = [0, len(T) - 1]
+        assert int(splits[-2]) * w.V < 2 ** 31 < int(splits[-1]) * w.V
     xs = torch.cat([x[splits[b]:splits[b + 1]] for b in pick]).cpu().numpy()
     tgs = np.ascontiguousarray(tg[pick][:, :max(int(U[pick].max()), 0)])
     s32, g32 = oracle.compute_transducer_loss(xs.copy(), tgs, T[pick], U[pick], w.blank, fls, osf)
-    s64, g64 = oracle.compute_transducer_loss(xs.copy(), tgs, T[pick], U[pick], w.blank, fls, osf,
-                                              dtype=np.float64)
+    if huge:  # no float64 run at this size (memory, time)
+        s64, g64 = s32, None
+    else:
+        s64, g64 = oracle.compute_transducer_loss(xs.copy(), tgs, T[pick], U[pick], w.blank, fls,
+                                                  osf, dtype=np.float64)
 
     work = x.clone()
     scores, grad, st = cabi.transducer_loss(work, dtg, dT, dU, w.blank, fls, osf, max_u1,
@@ -439,7 +449,9 @@ def test_full_size_workloads(name, make, device):
     tol = helpers.lattice_noise_tolerance(g32, helpers.per_row(s32, T[pick], U[pick]))
     assert (np.abs(got_g - g32) <= tol).all(), np.abs(got_g - g32).max()
     # float64 arbiter: no further from the exact gradient than the fp32 reference arithmetic
-    assert np.abs(got_g - g64).max() <= 2 * np.abs(g32 - g64).max() + 1e-6
+    if g64 is not None:
+        assert np.abs(got_g - g64).max() <= 2 * np.abs(g32 - g64).max() + 1e-6
+    del xs, g32, g64, got_g
 
     # size-independent properties over the whole batch
     if fls:
@@ -453,7 +465,8 @@ def test_full_size_workloads(name, make, device):
         assert torch.equal(work, x)  # log-softmax input is never written
     else:
         rs = grad.sum(1).abs().max().item()
-        assert rs < 1e-3, rs  # rows of d loss / d logits sum to zero
+        # rows of d loss / d logits sum to zero, up to the fp32 noise of exponents of size |loss|
+        assert rs < 1e-5 + 4 * helpers.EPS32 * np.abs(scores_np).max(), rs
         assert grad.data_ptr() == work.data_ptr()
     # entries are probabilities up to the fp32 noise of exp(arguments of size |loss|)
     assert grad.abs().max().item() <= 1 + 64 * helpers.EPS32 * np.abs(scores_np).max()

@@ -63,6 +63,18 @@ class Workload:
         return x.contiguous()
 
 
+def beyond_int32(seed=6, one_sym_per_frame=False):
+    """Four utterances of T=1100, U=499 at V=1000: 2.2 million packed rows, 2.2e9 logits
+    (more than 2^31 elements, 8.8 GB), plus one degenerate utterance in front so that no
+    offset is a round number.  The lattice has 8 waves per workgroup."""
+    T = np.array([3, 1100, 1100, 1100, 1100], np.int64)
+    U = np.array([1, 499, 499, 499, 499], np.int64)
+    rng = np.random.default_rng(seed)
+    name = "beyond_int32_N5_V1000%s" % ("_modified" if one_sym_per_frame else "")
+    return Workload(name, T, U, _targets(rng, 5, U.max(), 1000), 1000, 0, False,
+                    one_sym_per_frame, "mean", 1.0, 0.0, seed)
+
+
 def _targets(rng, N, max_u, V, zipf=False):
     cols = max(int(max_u), 0)
     if zipf:
