@@ -393,6 +393,52 @@ def test_side_stream_and_unaligned_views(device):
     assert torch.equal(view2.grad, a.grad)
 
 
+def test_whole_path_replays_from_a_hip_graph(device):
+    # ot_transducer_loss neither allocates nor synchronises nor clears memory with a memset,
+    # so a caller can capture it once and replay it; every replay is checked against the
+    # eager result for the data that is in the buffers at that moment
+    import ctypes
+    rng = np.random.default_rng(41)
+    T, U, tg, x0 = helpers.random_batch(rng, 6, 40, 70, 48)   # two waves per lattice
+    tg = np.where(tg == 0, 1, tg).astype(np.int32)
+    N, rows, V = len(T), x0.shape[0], x0.shape[1]
+    dT, dU, dtg = _dev(T, device), _dev(U, device), _dev(tg, device)
+    L = cabi.lib()
+    nbytes = L.ot_workspace_bytes(ctypes.c_int32(N), ctypes.c_int64(rows))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    logits = torch.empty((rows, V), device=device)
+    scores = torch.empty(N, device=device)
+    status = torch.zeros(64, dtype=torch.uint8, device=device)
+
+    def launch():
+        cabi.check(L.ot_transducer_loss(
+            cabi.ptr(logits), cabi.ptr(dtg), cabi.ptr(dT), cabi.ptr(dU), ctypes.c_int32(N),
+            ctypes.c_int32(tg.shape[1]), ctypes.c_int64(rows), ctypes.c_int32(V), ctypes.c_int32(0),
+            ctypes.c_int32(0), ctypes.c_int32(0), ctypes.c_int32(int(U.max()) + 1),
+            ctypes.c_float(0.5), cabi.ptr(ws), ctypes.c_size_t(nbytes), cabi.ptr(scores),
+            cabi.ptr(logits), cabi.ptr(status), cabi.stream()))
+
+    inputs = [x0] + [rng.standard_normal(x0.shape).astype(np.float32) for _ in range(3)]
+    eager = []
+    for xi in inputs:
+        logits.copy_(_dev(xi, device))
+        launch()
+        torch.cuda.synchronize()
+        eager.append((scores.clone(), logits.clone()))
+
+    graph = torch.cuda.CUDAGraph()
+    logits.copy_(_dev(inputs[0], device))
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        launch()
+    for k in (1, 2, 3, 0, 2):
+        logits.copy_(_dev(inputs[k], device))   # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(scores, eager[k][0]) and torch.equal(logits, eager[k][1]), k
+
+
 # ------------------------------------------------------------------ full sizes
 FULL = [
     ("asr", lambda: workloads.asr_batch()),
