@@ -46,13 +46,13 @@ def make_workload(name):
     raise SystemExit("unknown workload %r" % name)
 
 
-def algorithmic_bytes(w):
-    """Bytes per launch each kernel has to move, per packed row of V floats."""
+def algorithmic_bytes(w, esize=4):
+    """Bytes per launch each kernel has to move, per packed row of V elements of esize bytes."""
     R, V = w.rows, w.V
     if w.from_log_softmax:
-        return {"gather": 16 * R, "alpha_beta": 24 * R, "grad_logsoftmax": (4 * V + 24) * R}
-    return {"lse_gather": (4 * V + 4 + 8) * R, "alpha_beta": 24 * R,
-            "grad_logits": (8 * V + 20) * R}
+        return {"gather": 16 * R, "alpha_beta": 24 * R, "grad_logsoftmax": (esize * V + 24) * R}
+    return {"lse_gather": (esize * V + 4 + 8) * R, "alpha_beta": 24 * R,
+            "grad_logits": (2 * esize * V + 20) * R}
 
 
 def cpu_baseline(w, logits_host, max_seconds=30.0):
@@ -202,6 +202,9 @@ def main():
     ap.add_argument("--loss-weight", type=float, default=1.0,
                     help="multiply the loss by this before backward (a weighted or scaled loss); "
                          "the headline figure uses 1")
+    ap.add_argument("--logits-dtype", default="f32", choices=["f32", "f16", "bf16"],
+                    help="element type of the logits; the headline figure uses f32 (the only type "
+                         "the reference accepts), f16/bf16 measure the half-precision addition")
     ap.add_argument("--op", default="loss", choices=["loss", "joiner"],
                     help="loss: the headline benchmark; joiner: the packed joiner input "
                          "(pack_joiner) forward + backward for the workload's lengths")
@@ -230,6 +233,10 @@ def main():
     K, W = args.steps, args.warmup
 
     pristine = w.logits_torch(dev)
+    esize = 4
+    if args.logits_dtype != "f32":
+        pristine = pristine.to(torch.float16 if args.logits_dtype == "f16" else torch.bfloat16)
+        esize = 2
     targets = torch.from_numpy(w.targets).to(dev)
     T = torch.from_numpy(w.logit_lengths).to(dev)
     U = torch.from_numpy(w.target_lengths).to(dev)
@@ -274,11 +281,13 @@ def main():
         "metric": "utterances/sec fwd+bwd loss at N=32,V=500 fp32; achieved HBM GB/s vs peak",
         "value": w.N * K / elapsed, "unit": "utterances/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": 1e3 * elapsed / K, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "vs_baseline": None,
+        "dtype": "f32" if esize == 4 else "f32 arithmetic on %s logits" % args.logits_dtype,
+        "data": "synthetic",
         "config": {"workload": w.name, "N": w.N, "V": w.V, "packed_rows": w.rows,
                    "from_log_softmax": w.from_log_softmax,
                    "one_sym_per_frame": w.one_sym_per_frame, "reduction": w.reduction,
-                   "logits_bytes": 4 * w.rows * w.V, "seed": w.seed},
+                   "logits_bytes": esize * w.rows * w.V, "seed": w.seed},
     }
     if args.defer_gradient or args.loss_weight != 1.0:
         out["config"]["defer_gradient"] = args.defer_gradient
@@ -297,7 +306,7 @@ def main():
         per = {}
         for name, ms in ext.take_profile():
             per.setdefault(name, []).append(ms)
-        alg = algorithmic_bytes(w)
+        alg = algorithmic_bytes(w, esize)
         kernels = {}
         for name, ms in per.items():
             # a large batch is processed in two parts (two launches per step of the
@@ -311,17 +320,19 @@ def main():
         achieved = kernels[dom]["achieved_GBps"]
         kernel_name = "grad_flat_kernel<%d,%s>" % (4 if w.V % 4 == 0 else 1,
                                                     "true" if w.from_log_softmax else "false")
+        if esize == 2:
+            kernel_name = "grad_flat_half_kernel"
         out["roofline"] = {"bound": "hbm", "kernel": kernel_name, "achieved": achieved,
                            "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                            "frac": achieved / HBM_PEAK_GBPS,
-                           "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, dom)),
+                           "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, dom)) if esize == 4 else None,
                            "kernel_ms_per_step": kernels[dom]["ms_per_step"],
                            "launches_per_step": kernels[dom]["launches_per_step"],
                            "algorithmic_bytes_per_step": alg[dom]}
         out["kernels"] = kernels
 
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(w, pristine.cpu())
+        out["cpu_baseline"] = cpu_baseline(w, pristine.float().cpu())
         out["speedup_vs_cpu"] = out["value"] / out["cpu_baseline"]["value"]
 
     print(json.dumps(out), flush=True)

@@ -271,6 +271,38 @@ int ot_joiner_unpack_grad(const float *grad_out, const float *enc,
                           void *workspace, size_t workspace_bytes,
                           float *grad_enc, float *grad_dec, void *stream);
 
+/* ---- half-precision logits (not in the reference, which takes float32 only,
+ * transducer-loss.cc:33) ----
+ *
+ * For a joiner that runs under mixed precision: the two passes over the
+ * (rows, V) array read (and, for the gradient, write) 2-byte elements, all
+ * arithmetic and every per-row array stay float32.  Use these two in place of
+ * ot_log_probs and ot_gradient_apply; row offsets, lattice and coefficients
+ * (ot_row_splits, ot_alpha_beta, ot_row_coefficients) are the float32 ones. */
+#define OT_DTYPE_F32 0
+#define OT_DTYPE_F16 1  /* IEEE binary16 */
+#define OT_DTYPE_BF16 2 /* bfloat16      */
+
+/* ot_log_probs for logits of `dtype` (OT_DTYPE_F16 or OT_DTYPE_BF16). */
+int ot_log_probs_half(const void *logits, int32_t dtype, const int32_t *targets,
+                      const int32_t *target_lengths, const int32_t *row_splits,
+                      int32_t N, int32_t targets_cols, int64_t rows, int32_t V,
+                      int32_t blank, int32_t from_log_softmax, float *den,
+                      float *lp, void *stream);
+
+/* ot_gradient_apply for logits and gradient of `dtype`; the gradient is
+ * rounded to nearest even.  device_factor may be NULL (see
+ * ot_gradient_apply_device_factor). */
+int ot_gradient_apply_half(const void *logits, int32_t dtype,
+                           const void *row_scratch, int64_t rows, int32_t V,
+                           int32_t from_log_softmax, float grad_scale,
+                           const float *device_factor, void *grad, void *stream);
+
+/* ot_scale_by_device_scalar for n elements of `dtype` (product rounded to
+ * nearest even). */
+int ot_scale_by_device_scalar_half(void *x, int32_t dtype, int64_t n,
+                                   const float *factor, void *stream);
+
 /* Plain device-to-device copy kernel of n floats; used to calibrate profiler
  * byte counters against a transfer of known size. */
 int ot_copy_floats(const float *src, float *dst, int64_t n, void *stream);

@@ -139,6 +139,13 @@ void check_batch_values(const torch::Tensor &logits, const torch::Tensor &target
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// OT_DTYPE_F16 / OT_DTYPE_BF16 for half-precision logits, OT_DTYPE_F32 for anything else
+inline int half_dtype(const torch::Tensor &t) {
+  if (t.scalar_type() == torch::kHalf) return OT_DTYPE_F16;
+  if (t.scalar_type() == torch::kBFloat16) return OT_DTYPE_BF16;
+  return OT_DTYPE_F32;
+}
+
 // With `coefficients` set, the (rows, V) gradient pass is left to
 // apply_deferred_gradient: the per-row coefficients go into a tensor of their own,
 // handed back through the pointer, and the returned gradient is None.
@@ -154,7 +161,10 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   torch::CheckedFrom checked_from = "ComputeTransducerLoss";
 
   // transducer-loss.cc:33-46, same order
-  torch::checkScalarType(checked_from, logits_arg, torch::kFloat);
+  // float32 as in the reference; float16 / bfloat16 logits are an addition (the
+  // two passes over (rows, V) then read 2-byte elements, everything else is float32)
+  const int dtype = half_dtype(logits);
+  if (dtype == OT_DTYPE_F32) torch::checkScalarType(checked_from, logits_arg, torch::kFloat);
   torch::checkScalarType(checked_from, targets_arg, torch::kInt32);
   torch::checkScalarType(checked_from, logit_lengths_arg, torch::kInt32);
   torch::checkScalarType(checked_from, target_lengths_arg, torch::kInt32);
@@ -225,7 +235,8 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   auto *alpha = reinterpret_cast<float *>(w + off_alpha);
   auto *beta = reinterpret_cast<float *>(w + off_beta);
 
-  const float *p_logits = logits.data_ptr<float>();
+  const void *p_logits = logits.data_ptr();
+  const float *p_logits32 = dtype == OT_DTYPE_F32 ? logits.data_ptr<float>() : nullptr;
   const int32_t *p_targets = S > 0 ? targets.data_ptr<int32_t>() : nullptr;
   const int32_t *p_T = logit_lengths.data_ptr<int32_t>();
   const int32_t *p_U = target_lengths.data_ptr<int32_t>();
@@ -257,7 +268,8 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   //   main:  lse[rows < h]  lse[rows >= h]        grad[part A]      grad[part B]
   //   side:                 lattice+coeff[A]      lattice+coeff[B]
   // h is a row count, part A = the utterances that end at or before row h.
-  const bool overlap = overlap_enabled() && N >= 2 && rows * V >= kOverlapMinElements;
+  const bool overlap = overlap_enabled() && dtype == OT_DTYPE_F32 && N >= 2 &&
+                       rows * V >= kOverlapMinElements;
   const int64_t half = overlap ? rows / 2 : rows;
   EventGuard lse_a_done, lse_b_done;
 
@@ -266,11 +278,18 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   const bool blank_ok = (0 <= blank && blank < V);
   if (blank_ok) {
     ScopedTimer timer(from_log_softmax ? "gather" : "lse_gather", stream);
-    OT_CHECK(ot_log_probs_range(p_logits, p_targets, p_U, row_splits, (int32_t)N, (int32_t)S, rows,
-                                (int32_t)V, blank, from_log_softmax, 0, half, den, lp, stream));
+    if (dtype != OT_DTYPE_F32) {
+      OT_CHECK(ot_log_probs_half(p_logits, dtype, p_targets, p_U, row_splits, (int32_t)N,
+                                 (int32_t)S, rows, (int32_t)V, blank, from_log_softmax, den, lp,
+                                 stream));
+    } else {
+      OT_CHECK(ot_log_probs_range(p_logits32, p_targets, p_U, row_splits, (int32_t)N, (int32_t)S,
+                                  rows, (int32_t)V, blank, from_log_softmax, 0, half, den, lp,
+                                  stream));
+    }
     if (overlap) {
       OT_CHECK_HIP(hipEventRecord(lse_a_done.ev, stream));
-      OT_CHECK(ot_log_probs_range(p_logits, p_targets, p_U, row_splits, (int32_t)N, (int32_t)S,
+      OT_CHECK(ot_log_probs_range(p_logits32, p_targets, p_U, row_splits, (int32_t)N, (int32_t)S,
                                   rows, (int32_t)V, blank, from_log_softmax, half, rows, den, lp,
                                   stream));
       OT_CHECK_HIP(hipEventRecord(lse_b_done.ev, stream));
@@ -297,7 +316,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
               "an utterance with T = ", st.logit_len_max, " and up to ", max_u1,
               " lattice columns is too large for the lattice kernel");
 
-  torch::Tensor scores = torch::empty({N}, logits.options());
+  torch::Tensor scores = torch::empty({N}, logits.options().dtype(torch::kFloat));
   torch::Tensor gradient;
   const bool want_grad = logits.requires_grad();
   if (want_grad && !defer) {
@@ -305,7 +324,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
     // cpu.cc:814 / cuda.cu:449: the logits buffer itself otherwise.
     gradient = from_log_softmax ? torch::empty_like(logits) : logits;
   }
-  float *p_grad = gradient.defined() ? gradient.data_ptr<float>() : nullptr;
+  void *p_grad = gradient.defined() ? gradient.data_ptr() : nullptr;
 
   // lattice + per-row coefficients of utterances [b0, b1) on stream `s`
   auto lattice_part = [&](int32_t b0, int32_t b1, hipStream_t s) {
@@ -326,9 +345,14 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   auto gradient_part = [&](int32_t b0, int32_t b1) {
     if (!p_grad) return;
     ScopedTimer timer(from_log_softmax ? "grad_logsoftmax" : "grad_logits", stream);
-    OT_CHECK(ot_gradient_apply_range(p_logits, coef, rows, (int32_t)V, from_log_softmax,
-                                     (float)grad_scale, splits_host[b0], splits_host[b1], p_grad,
-                                     stream));
+    if (dtype != OT_DTYPE_F32) {
+      OT_CHECK(ot_gradient_apply_half(p_logits, dtype, coef, rows, (int32_t)V, from_log_softmax,
+                                      (float)grad_scale, nullptr, p_grad, stream));
+      return;
+    }
+    OT_CHECK(ot_gradient_apply_range(p_logits32, coef, rows, (int32_t)V, from_log_softmax,
+                                     (float)grad_scale, splits_host[b0], splits_host[b1],
+                                     static_cast<float *>(p_grad), stream));
   };
 
   // part A = utterances that lie completely in rows [0, half)
@@ -398,9 +422,11 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_transducer_loss
 torch::Tensor apply_deferred_gradient(torch::Tensor &logits, const torch::Tensor &coefficients,
                                       bool from_log_softmax, double grad_scale,
                                       const torch::Tensor &loss_grad) {
-  TORCH_CHECK(logits.is_cuda() && logits.scalar_type() == torch::kFloat && logits.dim() == 2 &&
-                  logits.is_contiguous(),
-              "apply_deferred_gradient: logits must be a contiguous 2-D float32 HIP tensor");
+  const int dtype = half_dtype(logits);
+  TORCH_CHECK(logits.is_cuda() && (dtype != OT_DTYPE_F32 || logits.scalar_type() == torch::kFloat) &&
+                  logits.dim() == 2 && logits.is_contiguous(),
+              "apply_deferred_gradient: logits must be a contiguous 2-D float32, float16 or "
+              "bfloat16 HIP tensor");
   const int64_t rows = logits.size(0), V = logits.size(1);
   TORCH_CHECK(rows > 0 && V > 0 && rows <= INT32_MAX && V <= INT32_MAX,
               "apply_deferred_gradient: bad logits shape");
@@ -415,6 +441,12 @@ torch::Tensor apply_deferred_gradient(torch::Tensor &logits, const torch::Tensor
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
   torch::Tensor gradient = from_log_softmax ? torch::empty_like(logits) : logits;
   ScopedTimer timer(from_log_softmax ? "grad_logsoftmax" : "grad_logits", stream);
+  if (dtype != OT_DTYPE_F32) {
+    OT_CHECK(ot_gradient_apply_half(logits.data_ptr(), dtype, coefficients.data_ptr(), rows,
+                                    (int32_t)V, from_log_softmax, (float)grad_scale,
+                                    loss_grad.data_ptr<float>(), gradient.data_ptr(), stream));
+    return gradient;
+  }
   OT_CHECK(ot_gradient_apply_device_factor(logits.data_ptr<float>(), coefficients.data_ptr(), rows,
                                            (int32_t)V, from_log_softmax, (float)grad_scale,
                                            loss_grad.data_ptr<float>(),
@@ -442,13 +474,20 @@ torch::Tensor negative_sum(const torch::Tensor &scores, double scale) {
 void scale_by_device_scalar_(torch::Tensor &x, const torch::Tensor &factor) {
   TORCH_CHECK(x.is_cuda() && factor.is_cuda() && x.device() == factor.device(),
               "scale_by_device_scalar_: both tensors must be on the same HIP device");
-  TORCH_CHECK(x.scalar_type() == torch::kFloat && factor.scalar_type() == torch::kFloat,
-              "scale_by_device_scalar_: float32 only");
+  const int dtype = half_dtype(x);
+  TORCH_CHECK((dtype != OT_DTYPE_F32 || x.scalar_type() == torch::kFloat) &&
+                  factor.scalar_type() == torch::kFloat,
+              "scale_by_device_scalar_: x must be float32, float16 or bfloat16 and factor float32");
   TORCH_CHECK(x.is_contiguous() && factor.numel() == 1,
               "scale_by_device_scalar_: x must be contiguous and factor a single element");
   c10::hip::HIPGuardMasqueradingAsCUDA device_guard(x.device());
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
   ScopedTimer timer("scale", stream);
+  if (dtype != OT_DTYPE_F32) {
+    OT_CHECK(ot_scale_by_device_scalar_half(x.data_ptr(), dtype, x.numel(),
+                                            factor.data_ptr<float>(), stream));
+    return;
+  }
   OT_CHECK(ot_scale_by_device_scalar(x.data_ptr<float>(), x.numel(), factor.data_ptr<float>(),
                                      stream));
 }

@@ -198,6 +198,9 @@ __device__ __forceinline__ Cell decode_row(const BlockUtterances &bu, int64_t ro
   return c;
 }
 
+// first column index of a row's gradient coefficients that marks an all-zero row
+constexpr int kZeroRow = -2;
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 // cache-policy operand of the raw buffer builtins: bit 1 = non-temporal

@@ -1,0 +1,406 @@
+// Half-precision logits (float16 / bfloat16) for the transducer loss: the two
+// kernels that touch the (rows, V) array, with float32 arithmetic inside.
+//
+// The reference accepts float32 logits only (transducer-loss.cc:33); a caller
+// whose joiner runs under mixed precision has to cast first.  Reading the
+// 2-byte logits directly halves the traffic of both streaming passes.  Every
+// per-row quantity (denominators, log-probabilities, alpha, beta, the gradient
+// coefficients) stays float32 and goes through the float32 kernels; only
+//   lse_gather_half_kernel   per-row log-sum-exp + blank/target gather
+//   gather_half_kernel       gather only (log-softmax input)
+//   grad_flat_half_kernel    (rows, V) gradient pass, in place for logits input
+// are specific to the element type.  Rows start at multiples of V elements, so
+// the access width is the largest of 8, 4, 2, 1 elements that divides V.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ot_device.hip.h"
+#include "ot_transducer.h"
+
+namespace ot {
+
+struct F16 {};   // IEEE binary16
+struct BF16 {};  // bfloat16: the upper half of a float32
+
+template <class E> __device__ __forceinline__ float to_float(unsigned short bits);
+template <> __device__ __forceinline__ float to_float<F16>(unsigned short bits) {
+  return (float)__builtin_bit_cast(_Float16, bits);
+}
+template <> __device__ __forceinline__ float to_float<BF16>(unsigned short bits) {
+  return __builtin_bit_cast(float, (unsigned)bits << 16);
+}
+template <class E> __device__ __forceinline__ unsigned short from_float(float x);
+template <> __device__ __forceinline__ unsigned short from_float<F16>(float x) {
+  return __builtin_bit_cast(unsigned short, (_Float16)x);  // round to nearest even
+}
+template <> __device__ __forceinline__ unsigned short from_float<BF16>(float x) {
+  return __builtin_bit_cast(unsigned short, (__bf16)x);  // round to nearest even
+}
+
+// VEC consecutive elements <-> floats; VEC * 2 bytes per access
+template <class E, int VEC> struct HalfIO {
+  static_assert(VEC == 1 || VEC == 2 || VEC == 4 || VEC == 8, "elements per access");
+  typedef unsigned short raw_t __attribute__((ext_vector_type(VEC)));
+  static __device__ __forceinline__ void load(const unsigned short *p, float (&v)[VEC]) {
+    raw_t r;
+    if (VEC == 1) r[0] = __builtin_nontemporal_load(p);
+    else r = __builtin_nontemporal_load(reinterpret_cast<const raw_t *>(p));
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) v[e] = to_float<E>(r[e]);
+  }
+  static __device__ __forceinline__ void store(unsigned short *p, const float (&v)[VEC]) {
+    raw_t r;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) r[e] = from_float<E>(v[e]);
+    if (VEC == 1) __builtin_nontemporal_store(r[0], p);
+    else __builtin_nontemporal_store(r, reinterpret_cast<raw_t *>(p));
+  }
+};
+
+// ---------------------------------------------------------------------------
+// per-row log-sum-exp + gather: one wave per row, kHalfRowsPerWave rows per wave,
+// RB of them in flight at a time
+// ---------------------------------------------------------------------------
+constexpr int kHalfRowsPerWave = 16;
+
+// K chunks of 64 * VEC elements cover a row (K = 0: any length, running maximum).
+// The wave first reduces its kHalfRowsPerWave rows, RB at a time, and keeps row r's
+// denominator in lane r; then lane pair (2r, 2r+1) gathers the blank and the target
+// value of row r, so that the dependent reads of the gather (row offsets, target,
+// logit) cost one round trip per wave instead of one per row.
+template <class E, int VEC, int K, int RB>
+__global__ __launch_bounds__(kBlock) void lse_gather_half_kernel(
+    const unsigned short *__restrict__ logits, const int32_t *__restrict__ targets,
+    const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits, int N,
+    int targets_cols, int64_t rows, int V, int blank, float *__restrict__ den,
+    float *__restrict__ lp) {
+  static_assert(2 * kHalfRowsPerWave <= kWave && kHalfRowsPerWave % RB == 0, "rows per wave");
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave_global = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  const int64_t row_first = wave_global * kHalfRowsPerWave;
+  if (row_first >= rows) return;
+  const int64_t row_end = min(rows, row_first + kHalfRowsPerWave);
+  constexpr int kChunk = kWave * VEC;
+  float dvec = 0.f;  // lane r: denominator of row row_first + r
+  if (K > 0) {
+    constexpr int KK = K > 0 ? K : 1;
+#pragma unroll
+    for (int r0 = 0; r0 < kHalfRowsPerWave; r0 += RB) {
+      if (row_first + r0 >= row_end) break;
+      float x[RB][KK][VEC];
+#pragma unroll
+      for (int r = 0; r < RB; ++r) {
+        const unsigned short *p = logits + min(row_first + r0 + r, row_end - 1) * (int64_t)V;
+#pragma unroll
+        for (int k = 0; k < KK; ++k) {
+          const int j = k * kChunk + lane * VEC;
+          if (j < V) {
+            HalfIO<E, VEC>::load(p + j, x[r][k]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) x[r][k][e] = OT_NEG_INF;
+          }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < RB; ++r) {
+        float cm = OT_NEG_INF;
+#pragma unroll
+        for (int k = 0; k < KK; ++k)
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) cm = fmaxf(cm, x[r][k][e]);
+        float m = group_allreduce<kWave>(cm, MaxOp());
+        if (__builtin_isinf(m)) m = 0.f;  // as ATen's logsumexp does for an all -inf / +inf row
+        float acc = 0.f;
+#pragma unroll
+        for (int k = 0; k < KK; ++k)
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc += exp_fast(x[r][k][e] - m);
+        const float s = group_allreduce<kWave>(acc, SumOp());
+        const float d = logf(s) + m;
+        dvec = (lane == r0 + r) ? d : dvec;
+      }
+    }
+  } else {
+    for (int r = 0; row_first + r < row_end; ++r) {
+      const unsigned short *p = logits + (row_first + r) * (int64_t)V;
+      float lm = OT_NEG_INF, ls = 0.f;
+      for (int j = lane * VEC; j < V; j += kChunk) {
+        float x[VEC];
+        HalfIO<E, VEC>::load(p + j, x);
+        float cm = OT_NEG_INF;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) cm = fmaxf(cm, x[e]);
+        const float nm = fmaxf(lm, cm);
+        const float ref = __builtin_isinf(nm) ? 0.f : nm;
+        float acc = (ls == 0.f) ? 0.f : ls * exp_fast((__builtin_isinf(lm) ? 0.f : lm) - ref);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc += exp_fast(x[e] - ref);
+        ls = acc;
+        lm = nm;
+      }
+      float m = group_allreduce<kWave>(lm, MaxOp());
+      if (__builtin_isinf(m)) m = 0.f;
+      const float lref = __builtin_isinf(lm) ? 0.f : lm;
+      const float part = (ls == 0.f) ? 0.f : ls * exp_fast(lref - m);
+      const float s = group_allreduce<kWave>(part, SumOp());
+      const float d = logf(s) + m;
+      dvec = (lane == r) ? d : dvec;
+    }
+  }
+
+  // denominators: lanes 0..15, one contiguous piece
+  if (row_first + lane < row_end) den[row_first + lane] = dvec;
+  // gather: lane pair (2r, 2r+1) = (blank, target) of row r
+  const int r = lane >> 1, which = lane & 1;
+  const float d = __shfl(dvec, r, kWave);
+  const int64_t row = row_first + r;
+  const int64_t lattice_rows = row_splits[N];
+  if (lane < 2 * kHalfRowsPerWave && row < row_end && row < lattice_rows) {
+    const int b = find_utterance(row_splits, N, row);
+    const int U = target_lengths[b];
+    const int u = (int)(row - row_splits[b]) % (U + 1 > 0 ? U + 1 : 1);
+    int col = blank;
+    bool ok = true;
+    if (which == 1) {
+      ok = u < U && u < targets_cols;
+      if (ok) {
+        col = targets[(int64_t)b * targets_cols + u];
+        ok = (unsigned)col < (unsigned)V;
+      }
+    }
+    lp[2 * row + which] = ok ? to_float<E>(logits[row * (int64_t)V + col]) - d : OT_NEG_INF;
+  }
+}
+
+// log-softmax input: lp is the two gathered values themselves
+template <class E>
+__global__ __launch_bounds__(kBlock) void gather_half_kernel(
+    const unsigned short *__restrict__ logits, const int32_t *__restrict__ targets,
+    const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits, int N,
+    int targets_cols, int64_t rows, int V, int blank, float *__restrict__ lp) {
+  const int64_t lattice_rows = min(rows, (int64_t)row_splits[N]);
+  const int64_t row = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (row >= lattice_rows) return;
+  const unsigned short *p = logits + row * (int64_t)V;
+  const float bl = to_float<E>(p[blank]);
+  const int b = find_utterance(row_splits, N, row);
+  const int U = target_lengths[b];
+  const int u = (int)(row - row_splits[b]) % (U + 1 > 0 ? U + 1 : 1);
+  float sym = OT_NEG_INF;
+  if (u < U && u < targets_cols) {
+    const int col = targets[(int64_t)b * targets_cols + u];
+    if ((unsigned)col < (unsigned)V) sym = to_float<E>(p[col]);
+  }
+  reinterpret_cast<float2 *>(lp)[row] = make_float2(bl, sym);
+}
+
+// ---------------------------------------------------------------------------
+// gradient: flat pass in units of VEC elements (VEC divides V: a unit never
+// straddles two rows); the per-row coefficients are those of row_coeff_kernel
+// ---------------------------------------------------------------------------
+constexpr int kHalfGradUnroll = 2;
+
+template <class E, int VEC, bool FLS>
+__global__ __launch_bounds__(kBlock) void grad_flat_half_kernel(
+    const unsigned short *logits, unsigned short *grad, const float4 *__restrict__ coef_f,
+    const int2 *__restrict__ coef_i, int64_t nunits, int nvec, float scale,
+    const float *__restrict__ device_factor) {
+  const float factor = device_factor ? *device_factor : 1.f;
+  if (!FLS) scale *= factor;
+#pragma unroll
+  for (int k = 0; k < kHalfGradUnroll; ++k) {
+    const int64_t unit = ((int64_t)blockIdx.x * kHalfGradUnroll + k) * kBlock + threadIdx.x;
+    if (unit >= nunits) return;
+    const int64_t row = unit / nvec;
+    const int col0 = (int)(unit - row * nvec) * VEC;
+    const float4 f = coef_f[row];
+    const int2 ci = coef_i[row];
+    float y[VEC];
+    if (FLS) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        y[e] = 0.f;
+        if (ci.x == col0 + e) y[e] = f.x * factor;
+        if (ci.y == col0 + e) y[e] = f.y * factor;
+      }
+    } else {
+      float x[VEC];
+      HalfIO<E, VEC>::load(logits + unit * VEC, x);
+      const bool zero = ci.x == kZeroRow;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        y[e] = zero ? 0.f : exp_any((x[e] + f.x) + f.y);
+        if (ci.x == col0 + e) y[e] -= exp_any((x[e] + f.x) + f.z);
+        if (ci.y == col0 + e) y[e] -= exp_any((x[e] + f.x) + f.w);
+        y[e] *= scale;
+      }
+    }
+    HalfIO<E, VEC>::store(grad + unit * VEC, y);
+  }
+}
+
+// x *= *factor for 2-byte elements, skipped on the device when *factor == 1
+template <class E>
+__global__ __launch_bounds__(kBlock) void scale_half_kernel(unsigned short *__restrict__ x,
+                                                            int64_t n,
+                                                            const float *__restrict__ factor) {
+  const float f = *factor;
+  if (f == 1.f) return;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    const int64_t n8 = n / 8;
+    for (int64_t i = tid; i < n8; i += stride) {
+      float v[8];
+      HalfIO<E, 8>::load(x + i * 8, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] *= f;
+      HalfIO<E, 8>::store(x + i * 8, v);
+    }
+    for (int64_t i = n8 * 8 + tid; i < n; i += stride) x[i] = from_float<E>(to_float<E>(x[i]) * f);
+  } else {
+    for (int64_t i = tid; i < n; i += stride) x[i] = from_float<E>(to_float<E>(x[i]) * f);
+  }
+}
+
+static inline int launch_status() { return (int)hipGetLastError(); }
+
+static inline int width_for(int V, const void *a, const void *b) {
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b);
+  int vec = 8;
+  while (vec > 1 && (V % vec != 0 || (bits & (uintptr_t)(vec * 2 - 1)) != 0)) vec >>= 1;
+  return vec;
+}
+
+template <class E>
+static int launch_log_probs(const unsigned short *logits, const int32_t *targets,
+                            const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
+                            int32_t targets_cols, int64_t rows, int32_t V, int32_t blank,
+                            int32_t from_log_softmax, float *den, float *lp, hipStream_t s) {
+  if (from_log_softmax) {
+    const unsigned blocks = (unsigned)((rows + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(gather_half_kernel<E>, dim3(blocks), dim3(kBlock), 0, s, logits, targets,
+                       target_lengths, row_splits, N, targets_cols, rows, V, blank, lp);
+    return launch_status();
+  }
+  const int vec = width_for(V, logits, nullptr);
+  const int64_t rows_per_block = (int64_t)kWavesPerBlock * kHalfRowsPerWave;
+  const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
+  const int chunks = (V + kWave * vec - 1) / (kWave * vec);
+  const int K = chunks <= 1 ? 1 : chunks <= 2 ? 2 : chunks <= 4 ? 4 : chunks <= 8 ? 8 : 0;
+#define OT_LAUNCH_LSEH(VEC_, K_, RB_)                                                              \
+  hipLaunchKernelGGL((lse_gather_half_kernel<E, VEC_, K_, RB_>), dim3(blocks), dim3(kBlock), 0, s, \
+                     logits, targets, target_lengths, row_splits, N, targets_cols, rows, V, blank,  \
+                     den, lp)
+#define OT_LAUNCH_LSEH_K(VEC_)                                                        \
+  switch (K) {                                                                        \
+    case 1: OT_LAUNCH_LSEH(VEC_, 1, 8); break;                                        \
+    case 2: OT_LAUNCH_LSEH(VEC_, 2, 4); break;                                        \
+    case 4: OT_LAUNCH_LSEH(VEC_, 4, 2); break;                                        \
+    case 8: OT_LAUNCH_LSEH(VEC_, 8, 1); break;                                        \
+    default: OT_LAUNCH_LSEH(VEC_, 0, 1); break;                                       \
+  }
+  switch (vec) {
+    case 8: OT_LAUNCH_LSEH_K(8) break;
+    case 4: OT_LAUNCH_LSEH_K(4) break;
+    case 2: OT_LAUNCH_LSEH_K(2) break;
+    default: OT_LAUNCH_LSEH_K(1) break;
+  }
+#undef OT_LAUNCH_LSEH_K
+#undef OT_LAUNCH_LSEH
+  return launch_status();
+}
+
+template <class E>
+static int launch_gradient(const unsigned short *logits, const void *row_scratch, int64_t rows,
+                           int32_t V, int32_t from_log_softmax, float grad_scale,
+                           const float *device_factor, unsigned short *grad, hipStream_t s) {
+  const float4 *coef_f = static_cast<const float4 *>(row_scratch);
+  const int2 *coef_i = reinterpret_cast<const int2 *>(coef_f + rows);
+  const int vec = width_for(V, grad, from_log_softmax ? nullptr : logits);
+  const int nvec = V / vec;
+  const int64_t nunits = rows * nvec;
+  const int64_t per_block = (int64_t)kHalfGradUnroll * kBlock;
+  const int64_t blocks = (nunits + per_block - 1) / per_block;
+  if (blocks > INT32_MAX) return OT_E_BAD_ARG;
+#define OT_LAUNCH_GRADH(VEC_, FLS_)                                                              \
+  hipLaunchKernelGGL((grad_flat_half_kernel<E, VEC_, FLS_>), dim3((unsigned)blocks), dim3(kBlock), \
+                     0, s, logits, grad, coef_f, coef_i, nunits, nvec, grad_scale, device_factor)
+#define OT_LAUNCH_GRADH_V(FLS_)                        \
+  switch (vec) {                                       \
+    case 8: OT_LAUNCH_GRADH(8, FLS_); break;           \
+    case 4: OT_LAUNCH_GRADH(4, FLS_); break;           \
+    case 2: OT_LAUNCH_GRADH(2, FLS_); break;           \
+    default: OT_LAUNCH_GRADH(1, FLS_); break;          \
+  }
+  if (from_log_softmax) { OT_LAUNCH_GRADH_V(true) } else { OT_LAUNCH_GRADH_V(false) }
+#undef OT_LAUNCH_GRADH_V
+#undef OT_LAUNCH_GRADH
+  return launch_status();
+}
+
+}  // namespace ot
+
+using namespace ot;
+
+extern "C" {
+
+int ot_log_probs_half(const void *logits, int32_t dtype, const int32_t *targets,
+                      const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
+                      int32_t targets_cols, int64_t rows, int32_t V, int32_t blank,
+                      int32_t from_log_softmax, float *den, float *lp, void *stream) {
+  if (!logits || !lp || !target_lengths || !row_splits || N <= 0 || rows <= 0 ||
+      rows > INT32_MAX || V <= 0 || blank < 0 || blank >= V || targets_cols < 0 ||
+      (targets_cols > 0 && !targets) || (!from_log_softmax && !den) ||
+      (dtype != OT_DTYPE_F16 && dtype != OT_DTYPE_BF16))
+    return OT_E_BAD_ARG;
+  if (reinterpret_cast<uintptr_t>(logits) & 1) return OT_E_MISALIGNED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned short *p = static_cast<const unsigned short *>(logits);
+  return dtype == OT_DTYPE_F16
+             ? launch_log_probs<F16>(p, targets, target_lengths, row_splits, N, targets_cols, rows,
+                                     V, blank, from_log_softmax, den, lp, s)
+             : launch_log_probs<BF16>(p, targets, target_lengths, row_splits, N, targets_cols, rows,
+                                      V, blank, from_log_softmax, den, lp, s);
+}
+
+int ot_gradient_apply_half(const void *logits, int32_t dtype, const void *row_scratch,
+                           int64_t rows, int32_t V, int32_t from_log_softmax, float grad_scale,
+                           const float *device_factor, void *grad, void *stream) {
+  if (!row_scratch || !grad || rows <= 0 || rows > INT32_MAX || V <= 0 ||
+      (dtype != OT_DTYPE_F16 && dtype != OT_DTYPE_BF16))
+    return OT_E_BAD_ARG;
+  if (from_log_softmax ? grad == logits : !logits) return OT_E_BAD_ARG;
+  if ((reinterpret_cast<uintptr_t>(grad) & 1) || (reinterpret_cast<uintptr_t>(logits) & 1) ||
+      (reinterpret_cast<uintptr_t>(row_scratch) & 15))
+    return OT_E_MISALIGNED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned short *p = static_cast<const unsigned short *>(logits);
+  unsigned short *g = static_cast<unsigned short *>(grad);
+  return dtype == OT_DTYPE_F16
+             ? launch_gradient<F16>(p, row_scratch, rows, V, from_log_softmax, grad_scale,
+                                    device_factor, g, s)
+             : launch_gradient<BF16>(p, row_scratch, rows, V, from_log_softmax, grad_scale,
+                                     device_factor, g, s);
+}
+
+int ot_scale_by_device_scalar_half(void *x, int32_t dtype, int64_t n, const float *factor,
+                                   void *stream) {
+  if (!x || !factor || n < 0 || (dtype != OT_DTYPE_F16 && dtype != OT_DTYPE_BF16))
+    return OT_E_BAD_ARG;
+  if (reinterpret_cast<uintptr_t>(x) & 1) return OT_E_MISALIGNED;
+  if (n == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int64_t blocks = (n / 8 + kBlock - 1) / kBlock;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks < 1) blocks = 1;
+  unsigned short *p = static_cast<unsigned short *>(x);
+  if (dtype == OT_DTYPE_F16)
+    hipLaunchKernelGGL(scale_half_kernel<F16>, dim3((unsigned)blocks), dim3(kBlock), 0, s, p, n, factor);
+  else
+    hipLaunchKernelGGL(scale_half_kernel<BF16>, dim3((unsigned)blocks), dim3(kBlock), 0, s, p, n, factor);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -674,7 +674,6 @@ __global__ __launch_bounds__(OT_MAX_U1) void alpha_beta_kernel(
 // tests before the target test, cpu.cc:514-523) decides which arc owns the
 // column when a target equals blank.  col1 == kZeroRow marks an all-zero row
 // (outside the one-symbol-per-frame band, or likelihood not finite).
-constexpr int kZeroRow = -2;
 
 template <bool FLS>
 __global__ __launch_bounds__(kBlock) void row_coeff_kernel(

@@ -16,7 +16,10 @@ Differences from the reference that do not change results:
 * ``TransducerLoss.__init__`` calls ``super().__init__()`` so the module can
   actually be called (the reference's class omits it, transducer_loss.py:173-188).
 
-One addition, off unless asked for: ``defer_gradient=True`` (keyword only) leaves
+Two additions.  ``logits`` may be float16 or bfloat16 (the reference takes
+float32 only, transducer-loss.cc:33): the passes over (rows, V) then read and
+write 2-byte elements, all arithmetic is float32, the loss is a float32 scalar
+and the gradient has the dtype of ``logits``.  And, off unless asked for: ``defer_gradient=True`` (keyword only) leaves
 ``logits`` untouched in ``forward`` and makes the single pass over (rows, V) in
 ``backward``, with ``loss_grad`` and ``1/N`` folded into it.  Results are the
 same; what changes is *when* ``logits`` is overwritten (in ``backward`` instead
@@ -117,6 +120,7 @@ class TransducerLossFunction(torch.autograd.Function):
             loss_grad.is_cuda
             and loss_grad.device == grad.device
             and loss_grad.dtype == torch.float32
+            and grad.dtype in (torch.float32, torch.float16, torch.bfloat16)
             and grad.is_contiguous()
         ):
             _optimized_transducer.scale_by_device_scalar_(grad, loss_grad.detach().contiguous())

@@ -186,3 +186,40 @@ def negative_sum(scores, scale):
     check(lib().ot_negative_sum(ptr(scores), ctypes.c_int32(scores.numel()), ctypes.c_float(scale),
                                 ptr(loss), stream()))
     return loss
+
+
+DTYPE = {torch.float16: 1, torch.bfloat16: 2}
+
+
+def log_probs_half(logits, targets, U, splits, blank, from_log_softmax):
+    rows, V = logits.shape
+    den = torch.full((rows,), float("nan"), dtype=torch.float32, device=logits.device)
+    lp = torch.full((rows, 2), float("nan"), dtype=torch.float32, device=logits.device)
+    cols = targets.shape[1]
+    check(lib().ot_log_probs_half(ptr(logits), ctypes.c_int32(DTYPE[logits.dtype]),
+                                  ptr(targets if cols else None), ptr(U), ptr(splits),
+                                  ctypes.c_int32(U.numel()), ctypes.c_int32(cols),
+                                  ctypes.c_int64(rows), ctypes.c_int32(V), ctypes.c_int32(blank),
+                                  ctypes.c_int32(int(from_log_softmax)), ptr(den), ptr(lp), stream()))
+    return den, lp
+
+
+def gradient_half(logits, lp, den, alpha, beta, targets, T, U, splits, blank, from_log_softmax,
+                  one_sym_per_frame, grad_scale=1.0, grad=None, device_factor=None):
+    """ot_row_coefficients (float32) + ot_gradient_apply_half."""
+    rows, V = logits.shape
+    if grad is None:
+        grad = torch.full((rows, V), float("nan"), dtype=logits.dtype, device=logits.device)
+    cols = targets.shape[1]
+    scratch = torch.empty(lib().ot_gradient_scratch_bytes(ctypes.c_int64(rows)), dtype=torch.uint8,
+                          device=logits.device)
+    check(lib().ot_row_coefficients(
+        ptr(lp), ptr(den), ptr(alpha), ptr(beta), ptr(targets if cols else None), ptr(T), ptr(U),
+        ptr(splits), ctypes.c_int32(T.numel()), ctypes.c_int32(cols), ctypes.c_int64(rows),
+        ctypes.c_int32(blank), ctypes.c_int32(int(from_log_softmax)),
+        ctypes.c_int32(int(one_sym_per_frame)), ctypes.c_float(grad_scale), ptr(scratch), stream()))
+    check(lib().ot_gradient_apply_half(
+        ptr(logits), ctypes.c_int32(DTYPE[logits.dtype]), ptr(scratch), ctypes.c_int64(rows),
+        ctypes.c_int32(V), ctypes.c_int32(int(from_log_softmax)), ctypes.c_float(grad_scale),
+        ptr(device_factor), ptr(grad), stream()))
+    return grad
