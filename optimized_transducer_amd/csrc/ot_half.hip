@@ -48,6 +48,15 @@ template <class E, int VEC> struct HalfIO {
 #pragma unroll
     for (int e = 0; e < VEC; ++e) v[e] = to_float<E>(r[e]);
   }
+  // ordinary load: for row pieces that share cache lines with their neighbours, where
+  // the non-temporal hint costs 20 %
+  static __device__ __forceinline__ void load_cached(const unsigned short *p, float (&v)[VEC]) {
+    raw_t r;
+    if (VEC == 1) r[0] = *p;
+    else r = *reinterpret_cast<const raw_t *>(p);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) v[e] = to_float<E>(r[e]);
+  }
   static __device__ __forceinline__ void store(unsigned short *p, const float (&v)[VEC]) {
     raw_t r;
 #pragma unroll
@@ -63,71 +72,74 @@ template <class E, int VEC> struct HalfIO {
 // ---------------------------------------------------------------------------
 constexpr int kHalfRowsPerWave = 16;
 
-// K chunks of 64 * VEC elements cover a row (K = 0: any length, running maximum).
-// The wave first reduces its kHalfRowsPerWave rows, RB at a time, and keeps row r's
-// denominator in lane r; then lane pair (2r, 2r+1) gathers the blank and the target
-// value of row r, so that the dependent reads of the gather (row offsets, target,
-// logit) cost one round trip per wave instead of one per row.
-template <class E, int VEC, int K, int RB>
+// A group of L lanes reduces one row (L * kHalfK * VEC >= V), so a wave reduces
+// 64 / L rows per pass with DPP butterflies; L = 0 stands for rows of any length
+// (whole wave per row, running maximum).  The wave first reduces its
+// kHalfRowsPerWave rows and keeps row r's denominator in lane r; then lane pair
+// (2r, 2r+1) gathers the blank and the target value of row r, so that the
+// dependent reads of the gather (row offsets, target, logit) cost one round trip
+// per wave instead of one per row.
+constexpr int kHalfK = 8;  // accesses per lane and row
+
+template <class E, int VEC, int L>
 __global__ __launch_bounds__(kBlock) void lse_gather_half_kernel(
     const unsigned short *__restrict__ logits, const int32_t *__restrict__ targets,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits, int N,
     int targets_cols, int64_t rows, int V, int blank, float *__restrict__ den,
     float *__restrict__ lp) {
-  static_assert(2 * kHalfRowsPerWave <= kWave && kHalfRowsPerWave % RB == 0, "rows per wave");
+  static_assert(2 * kHalfRowsPerWave <= kWave, "rows per wave");
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t wave_global = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
   const int64_t row_first = wave_global * kHalfRowsPerWave;
   if (row_first >= rows) return;
   const int64_t row_end = min(rows, row_first + kHalfRowsPerWave);
-  constexpr int kChunk = kWave * VEC;
   float dvec = 0.f;  // lane r: denominator of row row_first + r
-  if (K > 0) {
-    constexpr int KK = K > 0 ? K : 1;
-#pragma unroll
-    for (int r0 = 0; r0 < kHalfRowsPerWave; r0 += RB) {
+  if (L > 0) {
+    constexpr int LL = L > 0 ? L : kWave;
+    constexpr int G = kWave / LL;
+    static_assert(kHalfRowsPerWave % G == 0, "rows per pass");
+    const int sub = lane % LL, g = lane / LL;
+#pragma unroll 2
+    for (int r0 = 0; r0 < kHalfRowsPerWave; r0 += G) {
       if (row_first + r0 >= row_end) break;
-      float x[RB][KK][VEC];
+      const unsigned short *p = logits + min(row_first + r0 + g, row_end - 1) * (int64_t)V;
+      float x[kHalfK][VEC];
+      float cm = OT_NEG_INF;
 #pragma unroll
-      for (int r = 0; r < RB; ++r) {
-        const unsigned short *p = logits + min(row_first + r0 + r, row_end - 1) * (int64_t)V;
+      for (int k = 0; k < kHalfK; ++k) {
+        const int j = (k * LL + sub) * VEC;
+        if (j < V) {
+          HalfIO<E, VEC>::load_cached(p + j, x[k]);
+        } else {
 #pragma unroll
-        for (int k = 0; k < KK; ++k) {
-          const int j = k * kChunk + lane * VEC;
-          if (j < V) {
-            HalfIO<E, VEC>::load(p + j, x[r][k]);
-          } else {
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) x[r][k][e] = OT_NEG_INF;
-          }
+          for (int e = 0; e < VEC; ++e) x[k][e] = OT_NEG_INF;
         }
       }
 #pragma unroll
-      for (int r = 0; r < RB; ++r) {
-        float cm = OT_NEG_INF;
+      for (int k = 0; k < kHalfK; ++k)
 #pragma unroll
-        for (int k = 0; k < KK; ++k)
+        for (int e = 0; e < VEC; ++e) cm = fmaxf(cm, x[k][e]);
+      float m = group_allreduce<LL>(cm, MaxOp());
+      if (__builtin_isinf(m)) m = 0.f;  // as ATen's logsumexp does for an all -inf / +inf row
+      float acc = 0.f;
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) cm = fmaxf(cm, x[r][k][e]);
-        float m = group_allreduce<kWave>(cm, MaxOp());
-        if (__builtin_isinf(m)) m = 0.f;  // as ATen's logsumexp does for an all -inf / +inf row
-        float acc = 0.f;
+      for (int k = 0; k < kHalfK; ++k)
 #pragma unroll
-        for (int k = 0; k < KK; ++k)
-#pragma unroll
-          for (int e = 0; e < VEC; ++e) acc += exp_fast(x[r][k][e] - m);
-        const float s = group_allreduce<kWave>(acc, SumOp());
-        const float d = logf(s) + m;
-        dvec = (lane == r0 + r) ? d : dvec;
-      }
+        for (int e = 0; e < VEC; ++e) acc += exp_fast(x[k][e] - m);
+      const float s = group_allreduce<LL>(acc, SumOp());
+      const float d = logf(s) + m;
+      // lane r0 + i takes the result of group i
+      const float t = __shfl(d, ((lane - r0) & (G - 1)) * LL, kWave);
+      dvec = (lane >= r0 && lane < r0 + G) ? t : dvec;
     }
   } else {
+    constexpr int kChunk = kWave * VEC;
     for (int r = 0; row_first + r < row_end; ++r) {
       const unsigned short *p = logits + (row_first + r) * (int64_t)V;
       float lm = OT_NEG_INF, ls = 0.f;
       for (int j = lane * VEC; j < V; j += kChunk) {
         float x[VEC];
-        HalfIO<E, VEC>::load(p + j, x);
+        HalfIO<E, VEC>::load_cached(p + j, x);
         float cm = OT_NEG_INF;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) cm = fmaxf(cm, x[e]);
@@ -149,8 +161,8 @@ __global__ __launch_bounds__(kBlock) void lse_gather_half_kernel(
     }
   }
 
-  // denominators: lanes 0..15, one contiguous piece
-  if (row_first + lane < row_end) den[row_first + lane] = dvec;
+  // denominators: the first lanes, one contiguous piece
+  if (lane < kHalfRowsPerWave && row_first + lane < row_end) den[row_first + lane] = dvec;
   // gather: lane pair (2r, 2r+1) = (blank, target) of row r
   const int r = lane >> 1, which = lane & 1;
   const float d = __shfl(dvec, r, kWave);
@@ -287,19 +299,22 @@ static int launch_log_probs(const unsigned short *logits, const int32_t *targets
   const int vec = width_for(V, logits, nullptr);
   const int64_t rows_per_block = (int64_t)kWavesPerBlock * kHalfRowsPerWave;
   const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
-  const int chunks = (V + kWave * vec - 1) / (kWave * vec);
-  const int K = chunks <= 1 ? 1 : chunks <= 2 ? 2 : chunks <= 4 ? 4 : chunks <= 8 ? 8 : 0;
-#define OT_LAUNCH_LSEH(VEC_, K_, RB_)                                                              \
-  hipLaunchKernelGGL((lse_gather_half_kernel<E, VEC_, K_, RB_>), dim3(blocks), dim3(kBlock), 0, s, \
-                     logits, targets, target_lengths, row_splits, N, targets_cols, rows, V, blank,  \
+  // lanes per row: the smallest of 8, 16, 32, 64 with L * kHalfK accesses covering a row
+  const int nunits = (V + vec - 1) / vec;
+  int L = 8;
+  while (L < kWave && L * kHalfK < nunits) L *= 2;
+  if (L * kHalfK < nunits) L = 0;
+#define OT_LAUNCH_LSEH(VEC_, L_)                                                                  \
+  hipLaunchKernelGGL((lse_gather_half_kernel<E, VEC_, L_>), dim3(blocks), dim3(kBlock), 0, s,     \
+                     logits, targets, target_lengths, row_splits, N, targets_cols, rows, V, blank, \
                      den, lp)
 #define OT_LAUNCH_LSEH_K(VEC_)                                                        \
-  switch (K) {                                                                        \
-    case 1: OT_LAUNCH_LSEH(VEC_, 1, 8); break;                                        \
-    case 2: OT_LAUNCH_LSEH(VEC_, 2, 4); break;                                        \
-    case 4: OT_LAUNCH_LSEH(VEC_, 4, 2); break;                                        \
-    case 8: OT_LAUNCH_LSEH(VEC_, 8, 1); break;                                        \
-    default: OT_LAUNCH_LSEH(VEC_, 0, 1); break;                                       \
+  switch (L) {                                                                        \
+    case 8: OT_LAUNCH_LSEH(VEC_, 8); break;                                           \
+    case 16: OT_LAUNCH_LSEH(VEC_, 16); break;                                         \
+    case 32: OT_LAUNCH_LSEH(VEC_, 32); break;                                         \
+    case 64: OT_LAUNCH_LSEH(VEC_, 64); break;                                         \
+    default: OT_LAUNCH_LSEH(VEC_, 0); break;                                          \
   }
   switch (vec) {
     case 8: OT_LAUNCH_LSEH_K(8) break;
