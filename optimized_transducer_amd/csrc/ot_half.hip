@@ -208,13 +208,118 @@ __global__ __launch_bounds__(kBlock) void gather_half_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// gradient: flat pass in units of VEC elements (VEC divides V: a unit never
-// straddles two rows); the per-row coefficients are those of row_coeff_kernel
+// gradient: flat pass over the (rows, V) array, 16 bytes (8 elements) per access
+// whatever V is.  S = the largest of 8, 4, 2, 1 that divides V: S consecutive
+// elements that start at a multiple of S lie in one row, so an access is
+// 8 / S pieces, each with its own row (a 2V-byte row need not be a multiple of
+// 16 bytes).  The per-row coefficients are those of row_coeff_kernel.
 // ---------------------------------------------------------------------------
-constexpr int kHalfGradUnroll = 2;
+constexpr int kHalfGradUnroll = 2;  // accesses per thread
+constexpr int kHalfWide = 8;        // elements per access
 
-template <class E, int VEC, bool FLS>
+// gradient of S consecutive elements of one row, columns col0 .. col0 + S - 1
+template <int S, bool FLS>
+__device__ __forceinline__ void grad_piece(const float *x, float *y, const float4 f, const int2 ci,
+                                           int col0, float scale, float factor) {
+  // the two special columns are rarely among these S: one test for the piece
+  const unsigned d1 = (unsigned)(ci.x - col0), d2 = (unsigned)(ci.y - col0);
+  const bool special = d1 < (unsigned)S || d2 < (unsigned)S;
+  if (FLS) {
+#pragma unroll
+    for (int e = 0; e < S; ++e) y[e] = 0.f;
+    if (special) {
+#pragma unroll
+      for (int e = 0; e < S; ++e) {
+        if (d1 == (unsigned)e) y[e] = f.x * factor;
+        if (d2 == (unsigned)e) y[e] = f.y * factor;
+      }
+    }
+  } else {
+    const bool zero = ci.x == kZeroRow;
+#pragma unroll
+    for (int e = 0; e < S; ++e) y[e] = zero ? 0.f : exp_any((x[e] + f.x) + f.y);
+    if (special) {
+#pragma unroll
+      for (int e = 0; e < S; ++e) {
+        if (d1 == (unsigned)e) y[e] -= exp_any((x[e] + f.x) + f.z);
+        if (d2 == (unsigned)e) y[e] -= exp_any((x[e] + f.x) + f.w);
+      }
+    }
+    if (scale != 1.f) {
+#pragma unroll
+      for (int e = 0; e < S; ++e) y[e] *= scale;
+    }
+  }
+}
+
+template <class E, int S, bool FLS>
 __global__ __launch_bounds__(kBlock) void grad_flat_half_kernel(
+    const unsigned short *logits, unsigned short *grad, const float4 *__restrict__ coef_f,
+    const int2 *__restrict__ coef_i, int64_t total, int V, float inv_v, double inv_v_d,
+    float scale, const float *__restrict__ device_factor) {
+  const float factor = device_factor ? *device_factor : 1.f;
+  if (!FLS) scale *= factor;
+  constexpr int kPerBlock = kHalfGradUnroll * kBlock * kHalfWide;  // elements per workgroup
+  const int64_t base = (int64_t)blockIdx.x * kPerBlock;
+  // base / V through a double reciprocal (exact below 2^53) and one correction step
+  int64_t row_base = (int64_t)((double)base * inv_v_d);
+  {
+    const int64_t r = base - row_base * V;
+    if (r < 0) --row_base; else if (r >= V) ++row_base;
+  }
+  const int rem_base = (int)(base - row_base * V);
+  const int64_t wide_end = total - total % kHalfWide;  // whole 16-byte accesses end here
+  float x[kHalfGradUnroll][kHalfWide];
+#pragma unroll
+  for (int k = 0; k < kHalfGradUnroll; ++k) {
+    const int64_t elem = base + (int64_t)(k * kBlock + (int)threadIdx.x) * kHalfWide;
+    if (!FLS && elem < wide_end) HalfIO<E, kHalfWide>::load(logits + elem, x[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < kHalfGradUnroll; ++k) {
+    const int local = (k * kBlock + (int)threadIdx.x) * kHalfWide;
+    const int64_t elem = base + local;
+    if (elem >= wide_end) break;
+    float y[kHalfWide];
+    // row and column of the access's first element: idx < V + kPerBlock is exact in
+    // float, one correction step fixes the quotient; later pieces step to the next row
+    // when the column runs past V (S divides V: at most once per piece)
+    const int idx = rem_base + local;
+    int q = (int)((float)idx * inv_v);
+    if (q * V > idx) --q; else if ((q + 1) * V <= idx) ++q;
+    int col = idx - q * V;
+    int64_t row = row_base + q;
+    float4 f = coef_f[row];
+    int2 ci = coef_i[row];
+#pragma unroll
+    for (int j = 0; j < kHalfWide; j += S) {
+      if (col >= V) {
+        col -= V;
+        ++row;
+        f = coef_f[row];
+        ci = coef_i[row];
+      }
+      grad_piece<S, FLS>(&x[k][j], &y[j], f, ci, col, scale, factor);
+      col += S;
+    }
+    HalfIO<E, kHalfWide>::store(grad + elem, y);
+  }
+  // the last total % 8 elements (a multiple of S), S at a time
+  if (S < kHalfWide && blockIdx.x == gridDim.x - 1) {
+    const int64_t elem = wide_end + (int64_t)threadIdx.x * S;
+    if (elem < total) {
+      float xs[S], ys[S];
+      if (!FLS) HalfIO<E, S>::load(logits + elem, xs);
+      const int64_t row = elem / V;
+      grad_piece<S, FLS>(xs, ys, coef_f[row], coef_i[row], (int)(elem - row * V), scale, factor);
+      HalfIO<E, S>::store(grad + elem, ys);
+    }
+  }
+}
+
+// the same pass with S elements per access, for buffers that are not 16-byte aligned
+template <class E, int S, bool FLS>
+__global__ __launch_bounds__(kBlock) void grad_flat_half_narrow_kernel(
     const unsigned short *logits, unsigned short *grad, const float4 *__restrict__ coef_f,
     const int2 *__restrict__ coef_i, int64_t nunits, int nvec, float scale,
     const float *__restrict__ device_factor) {
@@ -225,30 +330,10 @@ __global__ __launch_bounds__(kBlock) void grad_flat_half_kernel(
     const int64_t unit = ((int64_t)blockIdx.x * kHalfGradUnroll + k) * kBlock + threadIdx.x;
     if (unit >= nunits) return;
     const int64_t row = unit / nvec;
-    const int col0 = (int)(unit - row * nvec) * VEC;
-    const float4 f = coef_f[row];
-    const int2 ci = coef_i[row];
-    float y[VEC];
-    if (FLS) {
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        y[e] = 0.f;
-        if (ci.x == col0 + e) y[e] = f.x * factor;
-        if (ci.y == col0 + e) y[e] = f.y * factor;
-      }
-    } else {
-      float x[VEC];
-      HalfIO<E, VEC>::load(logits + unit * VEC, x);
-      const bool zero = ci.x == kZeroRow;
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        y[e] = zero ? 0.f : exp_any((x[e] + f.x) + f.y);
-        if (ci.x == col0 + e) y[e] -= exp_any((x[e] + f.x) + f.z);
-        if (ci.y == col0 + e) y[e] -= exp_any((x[e] + f.x) + f.w);
-        y[e] *= scale;
-      }
-    }
-    HalfIO<E, VEC>::store(grad + unit * VEC, y);
+    float x[S], y[S];
+    if (!FLS) HalfIO<E, S>::load(logits + unit * S, x);
+    grad_piece<S, FLS>(x, y, coef_f[row], coef_i[row], (int)(unit - row * nvec) * S, scale, factor);
+    HalfIO<E, S>::store(grad + unit * S, y);
   }
 }
 
@@ -333,25 +418,52 @@ static int launch_gradient(const unsigned short *logits, const void *row_scratch
                            const float *device_factor, unsigned short *grad, hipStream_t s) {
   const float4 *coef_f = static_cast<const float4 *>(row_scratch);
   const int2 *coef_i = reinterpret_cast<const int2 *>(coef_f + rows);
-  const int vec = width_for(V, grad, from_log_softmax ? nullptr : logits);
-  const int nvec = V / vec;
-  const int64_t nunits = rows * nvec;
-  const int64_t per_block = (int64_t)kHalfGradUnroll * kBlock;
-  const int64_t blocks = (nunits + per_block - 1) / per_block;
-  if (blocks > INT32_MAX) return OT_E_BAD_ARG;
-#define OT_LAUNCH_GRADH(VEC_, FLS_)                                                              \
-  hipLaunchKernelGGL((grad_flat_half_kernel<E, VEC_, FLS_>), dim3((unsigned)blocks), dim3(kBlock), \
-                     0, s, logits, grad, coef_f, coef_i, nunits, nvec, grad_scale, device_factor)
-#define OT_LAUNCH_GRADH_V(FLS_)                        \
-  switch (vec) {                                       \
+  int S = 8;  // elements that never straddle two rows
+  while (S > 1 && V % S != 0) S >>= 1;
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(grad) |
+                         (from_log_softmax ? 0 : reinterpret_cast<uintptr_t>(logits));
+  const int64_t total = rows * (int64_t)V;
+  if ((bits & 15) == 0 && V < (1 << 23)) {
+    const int64_t per_block = (int64_t)kHalfGradUnroll * kBlock * kHalfWide;
+    const int64_t blocks = (total + per_block - 1) / per_block;
+    if (blocks > INT32_MAX) return OT_E_BAD_ARG;
+#define OT_LAUNCH_GRADH(S_, FLS_)                                                               \
+  hipLaunchKernelGGL((grad_flat_half_kernel<E, S_, FLS_>), dim3((unsigned)blocks), dim3(kBlock), \
+                     0, s, logits, grad, coef_f, coef_i, total, V, 1.0f / (float)V,             \
+                     1.0 / (double)V, grad_scale, device_factor)
+#define OT_LAUNCH_GRADH_S(FLS_)                        \
+  switch (S) {                                         \
     case 8: OT_LAUNCH_GRADH(8, FLS_); break;           \
     case 4: OT_LAUNCH_GRADH(4, FLS_); break;           \
     case 2: OT_LAUNCH_GRADH(2, FLS_); break;           \
     default: OT_LAUNCH_GRADH(1, FLS_); break;          \
   }
-  if (from_log_softmax) { OT_LAUNCH_GRADH_V(true) } else { OT_LAUNCH_GRADH_V(false) }
-#undef OT_LAUNCH_GRADH_V
+    if (from_log_softmax) { OT_LAUNCH_GRADH_S(true) } else { OT_LAUNCH_GRADH_S(false) }
+#undef OT_LAUNCH_GRADH_S
 #undef OT_LAUNCH_GRADH
+    return launch_status();
+  }
+  // narrow accesses: S limited by the alignment of the buffers as well
+  while (S > 1 && (bits & (uintptr_t)(S * 2 - 1)) != 0) S >>= 1;
+  const int nvec = V / S;
+  const int64_t nunits = rows * nvec;
+  const int64_t per_block = (int64_t)kHalfGradUnroll * kBlock;
+  const int64_t blocks = (nunits + per_block - 1) / per_block;
+  if (blocks > INT32_MAX) return OT_E_BAD_ARG;
+#define OT_LAUNCH_GRADN(S_, FLS_)                                                                \
+  hipLaunchKernelGGL((grad_flat_half_narrow_kernel<E, S_, FLS_>), dim3((unsigned)blocks),         \
+                     dim3(kBlock), 0, s, logits, grad, coef_f, coef_i, nunits, nvec, grad_scale,  \
+                     device_factor)
+#define OT_LAUNCH_GRADN_S(FLS_)                        \
+  switch (S) {                                         \
+    case 8: OT_LAUNCH_GRADN(8, FLS_); break;           \
+    case 4: OT_LAUNCH_GRADN(4, FLS_); break;           \
+    case 2: OT_LAUNCH_GRADN(2, FLS_); break;           \
+    default: OT_LAUNCH_GRADN(1, FLS_); break;          \
+  }
+  if (from_log_softmax) { OT_LAUNCH_GRADN_S(true) } else { OT_LAUNCH_GRADN_S(false) }
+#undef OT_LAUNCH_GRADN_S
+#undef OT_LAUNCH_GRADN
   return launch_status();
 }
 

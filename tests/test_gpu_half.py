@@ -75,6 +75,40 @@ def test_log_probs_and_gradient_kernels(V, dtype, device):
             buf = xin.clone()
             out = cabi.gradient_half(buf, *args[1:], grad=buf)
             assert out.data_ptr() == buf.data_ptr() and torch.equal(buf.float().cpu(), torch.from_numpy(got))
+            # a buffer that starts 2 bytes into an allocation: narrow accesses, same bits
+            flat = torch.zeros(xin.numel() + 1, dtype=dtype, device=device)
+            view = flat[1:].view(xin.shape)
+            view.copy_(xin)
+            cabi.gradient_half(view, *args[1:], grad=view)
+            assert torch.equal(view.float().cpu(), torch.from_numpy(got)) and flat[0].item() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f16", "bf16"])
+@pytest.mark.parametrize("V,rows_odd", [(20, True), (20, False), (6, True), (500, True), (9, True)])
+def test_gradient_kernel_tail_of_the_array(V, rows_odd, dtype, device):
+    # 16-byte accesses cover the array up to a multiple of 8 elements; the rest is done apart
+    T = np.array([3, 2 if rows_odd else 3], np.int32)
+    U = np.array([2, 1], np.int32)          # 9 + 4 = 13 rows, or 9 + 6 = 15 rows
+    if not rows_odd:
+        T[1], U[1] = 2, 2                   # 9 + 6 = 15 rows is odd too: make it 3*3 + 1*... even
+        T[0] = 2                            # 6 + 6 = 12 rows
+    rng = np.random.default_rng(V)
+    rows = int((T * (U + 1)).sum())
+    tg = rng.integers(1, V, size=(2, int(U.max()))).astype(np.int32)
+    xh = torch.from_numpy(rng.standard_normal((rows, V)).astype(np.float32)).to(dtype)
+    x32 = xh.float().numpy()
+    s, g, parts = helpers.oracle_full(x32, tg, T, U, 0, False, False)
+    ninf = lambda v: np.where(np.isnan(v), -np.inf, v).astype(np.float32)  # noqa: E731
+    dT, dU, dtg = _dev(T, device), _dev(U, device), _dev(tg, device)
+    splits, _ = cabi.row_splits(dT, dU, dtg)
+    buf = xh.to(device)
+    guard = torch.full((64,), 7.0, dtype=dtype, device=device)  # allocated right after, must survive
+    cabi.gradient_half(buf, _dev(ninf(parts["lp"]), device), _dev(parts["den"], device),
+                       _dev(ninf(parts["alpha"]), device), _dev(ninf(parts["beta"]), device), dtg, dT,
+                       dU, splits, 0, False, False, grad=buf)
+    got = buf.float().cpu().numpy()
+    assert (np.abs(got - g) <= ULP[dtype] * np.abs(g) + 1e-6).all(), np.abs(got - g).max()
+    assert (guard == 7.0).all()
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f16", "bf16"])
