@@ -72,6 +72,118 @@ template <class E, int VEC> struct HalfIO {
 // ---------------------------------------------------------------------------
 constexpr int kHalfRowsPerWave = 16;
 
+// Outputs of one wave's rows: dvec holds row r's denominator in lane r.  Lanes
+// 0..15 store the denominators as one contiguous piece; lane pair (2r, 2r+1)
+// gathers the blank and the target value of row r.
+template <class E>
+__device__ __forceinline__ void finish_rows(float dvec, int lane, int64_t row_first, int64_t row_end,
+                                            const unsigned short *__restrict__ logits,
+                                            const int32_t *__restrict__ targets,
+                                            const int32_t *__restrict__ target_lengths,
+                                            const int32_t *__restrict__ row_splits, int N,
+                                            int targets_cols, int V, int blank,
+                                            float *__restrict__ den, float *__restrict__ lp) {
+  if (lane < kHalfRowsPerWave && row_first + lane < row_end) den[row_first + lane] = dvec;
+  const int r = lane >> 1, which = lane & 1;
+  const float d = __shfl(dvec, r, kWave);
+  const int64_t row = row_first + r;
+  const int64_t lattice_rows = row_splits[N];
+  if (lane < 2 * kHalfRowsPerWave && row < row_end && row < lattice_rows) {
+    const int b = find_utterance(row_splits, N, row);
+    const int U = target_lengths[b];
+    const int u = (int)(row - row_splits[b]) % (U + 1 > 0 ? U + 1 : 1);
+    int col = blank;
+    bool ok = true;
+    if (which == 1) {
+      ok = u < U && u < targets_cols;
+      if (ok) {
+        col = targets[(int64_t)b * targets_cols + u];
+        ok = (unsigned)col < (unsigned)V;
+      }
+    }
+    lp[2 * row + which] = ok ? to_float<E>(logits[row * (int64_t)V + col]) - d : OT_NEG_INF;
+  }
+}
+
+// 8 elements of a 16-byte access
+template <class E>
+__device__ __forceinline__ void unpack8(u32x4 raw, float (&v)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = to_float<E>((unsigned short)(raw[i] & 0xffffu));
+    v[2 * i + 1] = to_float<E>((unsigned short)(raw[i] >> 16));
+  }
+}
+
+// Rows of 2V bytes start at any even byte offset.  For a 16-byte aligned array the
+// denominator pass still moves 16 aligned bytes per lane: a group of L lanes reads
+// the K * L aligned 16-byte pieces that cover its row, starting at the boundary at
+// or below the row's first byte, and elements of the neighbouring rows in the first
+// and the last piece are masked.  Ordinary (cached) loads: neighbouring rows share
+// those pieces.  The wave's rows are one raw buffer, so the last piece of the last
+// row may reach past the array: it reads zeros there, which are masked like the rest.
+template <class E, int L, int K>
+__global__ __launch_bounds__(kBlock) void lse_gather_half_wide_kernel(
+    const unsigned short *__restrict__ logits, const int32_t *__restrict__ targets,
+    const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits, int N,
+    int targets_cols, int64_t rows, int V, int blank, float *__restrict__ den,
+    float *__restrict__ lp) {
+  constexpr int G = kWave / L;
+  static_assert(kHalfRowsPerWave % G == 0, "rows per pass");
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave_global = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  const int64_t row_first = wave_global * kHalfRowsPerWave;
+  if (row_first >= rows) return;
+  const int64_t row_end = min(rows, row_first + kHalfRowsPerWave);
+  const int sub = lane % L, g = lane / L;
+  const unsigned row_bytes = (unsigned)V * 2u;
+  const int64_t byte0 = row_first * (int64_t)V * 2;
+  const unsigned shift = (unsigned)(byte0 & 15);
+  // size rounded up to whole dwords (the bounds check is per dword): with an odd number
+  // of elements the last one shares its aligned dword with two bytes past the array
+  const __amdgpu_buffer_rsrc_t buf =
+      make_buffer(reinterpret_cast<const char *>(logits) + (byte0 - shift),
+                  ((unsigned)(row_end - row_first) * row_bytes + shift + 3u) & ~3u);
+  float dvec = 0.f;
+  for (int r0 = 0; r0 < kHalfRowsPerWave; r0 += G) {
+    if (row_first + r0 >= row_end) break;
+    // bytes [rs, rs + row_bytes) of the buffer are this group's row (a row past the
+    // wave's last one lies past the buffer: every element masked or zero)
+    const unsigned rs = shift + (unsigned)(r0 + g) * row_bytes;
+    const unsigned a = rs & ~15u;
+    float x[K][8];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const unsigned off = a + (unsigned)(k * L + sub) * 16u;
+      unpack8<E>(__builtin_amdgcn_raw_buffer_load_b128(buf, off, 0, 0), x[k]);
+      const unsigned lo = rs - off;  // byte offset of the row's first element in this piece
+      if (off < rs || off + 16u > rs + row_bytes) {  // a piece at either end of the row
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          x[k][e] = ((unsigned)(2 * e) - lo < row_bytes) ? x[k][e] : OT_NEG_INF;
+      }
+    }
+    float cm = OT_NEG_INF;
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) cm = fmaxf(cm, x[k][e]);
+    float m = group_allreduce<L>(cm, MaxOp());
+    if (__builtin_isinf(m)) m = 0.f;  // as ATen's logsumexp does for an all -inf / +inf row
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += exp_fast(x[k][e] - m);
+    const float s = group_allreduce<L>(acc, SumOp());
+    const float d = logf(s) + m;
+    const float t = __shfl(d, ((lane - r0) & (G - 1)) * L, kWave);
+    dvec = (lane >= r0 && lane < r0 + G) ? t : dvec;
+  }
+  finish_rows<E>(dvec, lane, row_first, row_end, logits, targets, target_lengths, row_splits, N,
+                 targets_cols, V, blank, den, lp);
+}
+
 // A group of L lanes reduces one row (L * kHalfK * VEC >= V), so a wave reduces
 // 64 / L rows per pass with DPP butterflies; L = 0 stands for rows of any length
 // (whole wave per row, running maximum).  The wave first reduces its
@@ -161,28 +273,8 @@ __global__ __launch_bounds__(kBlock) void lse_gather_half_kernel(
     }
   }
 
-  // denominators: the first lanes, one contiguous piece
-  if (lane < kHalfRowsPerWave && row_first + lane < row_end) den[row_first + lane] = dvec;
-  // gather: lane pair (2r, 2r+1) = (blank, target) of row r
-  const int r = lane >> 1, which = lane & 1;
-  const float d = __shfl(dvec, r, kWave);
-  const int64_t row = row_first + r;
-  const int64_t lattice_rows = row_splits[N];
-  if (lane < 2 * kHalfRowsPerWave && row < row_end && row < lattice_rows) {
-    const int b = find_utterance(row_splits, N, row);
-    const int U = target_lengths[b];
-    const int u = (int)(row - row_splits[b]) % (U + 1 > 0 ? U + 1 : 1);
-    int col = blank;
-    bool ok = true;
-    if (which == 1) {
-      ok = u < U && u < targets_cols;
-      if (ok) {
-        col = targets[(int64_t)b * targets_cols + u];
-        ok = (unsigned)col < (unsigned)V;
-      }
-    }
-    lp[2 * row + which] = ok ? to_float<E>(logits[row * (int64_t)V + col]) - d : OT_NEG_INF;
-  }
+  finish_rows<E>(dvec, lane, row_first, row_end, logits, targets, target_lengths, row_splits, N,
+                 targets_cols, V, blank, den, lp);
 }
 
 // log-softmax input: lp is the two gathered values themselves
@@ -381,9 +473,34 @@ static int launch_log_probs(const unsigned short *logits, const int32_t *targets
                        target_lengths, row_splits, N, targets_cols, rows, V, blank, lp);
     return launch_status();
   }
-  const int vec = width_for(V, logits, nullptr);
   const int64_t rows_per_block = (int64_t)kWavesPerBlock * kHalfRowsPerWave;
   const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
+  if ((reinterpret_cast<uintptr_t>(logits) & 15) == 0) {
+    // aligned 16-byte pieces that cover a row wherever it starts
+    const int pieces = (V * 2) % 16 == 0 ? V / 8 : (V * 2 + 14 + 15) / 16;
+    const int K = pieces <= 4 * kWave ? 4 : 8;
+    int L = 8;
+    while (L < kWave && L * K < pieces) L *= 2;
+    if (L * K >= pieces) {
+#define OT_LAUNCH_LSEW(L_, K_)                                                                    \
+  hipLaunchKernelGGL((lse_gather_half_wide_kernel<E, L_, K_>), dim3(blocks), dim3(kBlock), 0, s,  \
+                     logits, targets, target_lengths, row_splits, N, targets_cols, rows, V, blank, \
+                     den, lp)
+      if (K == 4) {
+        switch (L) {
+          case 8: OT_LAUNCH_LSEW(8, 4); break;
+          case 16: OT_LAUNCH_LSEW(16, 4); break;
+          case 32: OT_LAUNCH_LSEW(32, 4); break;
+          default: OT_LAUNCH_LSEW(64, 4); break;
+        }
+      } else {
+        OT_LAUNCH_LSEW(64, 8);
+      }
+#undef OT_LAUNCH_LSEW
+      return launch_status();
+    }
+  }
+  const int vec = width_for(V, logits, nullptr);
   // lanes per row: the smallest of 8, 16, 32, 64 with L * kHalfK accesses covering a row
   const int nunits = (V + vec - 1) / vec;
   int L = 8;

@@ -50,6 +50,13 @@ def test_log_probs_and_gradient_kernels(V, dtype, device):
     m = ~np.isnan(wlp)
     got = lp.cpu().numpy()
     assert np.allclose(got[m], wlp[m], rtol=RTOL, atol=ATOL) and np.isneginf(got[~m]).all()
+    # logits that start 2 bytes into an allocation take the narrow-access kernel
+    flat = torch.zeros(xh.numel() + 1, dtype=dtype, device=device)
+    view = flat[1:].view(xh.shape)
+    view.copy_(xh)
+    den_v, lp_v = cabi.log_probs_half(view, dtg, dU, splits, 0, False)
+    assert (np.abs(den_v.cpu().numpy() - wden) <= 4 * ulp).all()
+    assert np.allclose(lp_v.cpu().numpy()[m], wlp[m], rtol=RTOL, atol=ATOL)
     # log-softmax input: pure gather, bit exact
     xl = torch.log_softmax(xh.float(), 1).to(dtype)
     _, lp2 = cabi.log_probs_half(xl, dtg, dU, splits, 0, True)
