@@ -303,13 +303,18 @@ __global__ __launch_bounds__(kBlock) void gather_half_kernel(
 // gradient: flat pass over the (rows, V) array, 16 bytes (8 elements) per access
 // whatever V is.  S = the largest of 8, 4, 2, 1 that divides V: S consecutive
 // elements that start at a multiple of S lie in one row, so an access is
-// 8 / S pieces, each with its own row (a 2V-byte row need not be a multiple of
-// 16 bytes).  The per-row coefficients are those of row_coeff_kernel.
+// 8 / S pieces; for V >= 8 they belong to at most two rows (a 2V-byte row need
+// not be a multiple of 16 bytes).  The per-row coefficients are those of
+// row_coeff_kernel.
 // ---------------------------------------------------------------------------
 constexpr int kHalfGradUnroll = 2;  // accesses per thread
 constexpr int kHalfWide = 8;        // elements per access
 
-// gradient of S consecutive elements of one row, columns col0 .. col0 + S - 1
+// Gradient of S consecutive elements of one row, columns col0 .. col0 + S - 1.
+// The result is rounded to 8 or 11 significant bits, so the common entries take
+// the one-multiply exponential (relative error 1e-7 + |argument| * 9e-8, below
+// 2e-7 absolute for values <= 1); the two special columns, where two terms may
+// cancel, keep the accurate one.
 template <int S, bool FLS>
 __device__ __forceinline__ void grad_piece(const float *x, float *y, const float4 f, const int2 ci,
                                            int col0, float scale, float factor) {
@@ -328,13 +333,17 @@ __device__ __forceinline__ void grad_piece(const float *x, float *y, const float
     }
   } else {
     const bool zero = ci.x == kZeroRow;
+    const float shift = f.x + f.y;
 #pragma unroll
-    for (int e = 0; e < S; ++e) y[e] = zero ? 0.f : exp_any((x[e] + f.x) + f.y);
+    for (int e = 0; e < S; ++e) {
+      const float v = exp_fast(x[e] + shift);
+      y[e] = zero ? 0.f : v;
+    }
     if (special) {
 #pragma unroll
       for (int e = 0; e < S; ++e) {
-        if (d1 == (unsigned)e) y[e] -= exp_any((x[e] + f.x) + f.z);
-        if (d2 == (unsigned)e) y[e] -= exp_any((x[e] + f.x) + f.w);
+        if (d1 == (unsigned)e) y[e] = exp_any((x[e] + f.x) + f.y) - exp_any((x[e] + f.x) + f.z);
+        if (d2 == (unsigned)e) y[e] = exp_any((x[e] + f.x) + f.y) - exp_any((x[e] + f.x) + f.w);
       }
     }
     if (scale != 1.f) {
@@ -344,11 +353,24 @@ __device__ __forceinline__ void grad_piece(const float *x, float *y, const float
   }
 }
 
+template <class E>
+__device__ __forceinline__ u32x4 pack8(const float (&v)[8]) {
+  u32x4 raw;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    raw[i] = (unsigned)from_float<E>(v[2 * i]) | ((unsigned)from_float<E>(v[2 * i + 1]) << 16);
+  return raw;
+}
+
+// V >= 8.  A workgroup owns kHalfGradUnroll * 256 consecutive 16-byte accesses as one
+// raw buffer (the tail of the last workgroup needs no branch); the coefficients of
+// the access's first row and of the row after it are both loaded up front, and each
+// piece picks one of the two without a branch.
 template <class E, int S, bool FLS>
 __global__ __launch_bounds__(kBlock) void grad_flat_half_kernel(
     const unsigned short *logits, unsigned short *grad, const float4 *__restrict__ coef_f,
-    const int2 *__restrict__ coef_i, int64_t total, int V, float inv_v, double inv_v_d,
-    float scale, const float *__restrict__ device_factor) {
+    const int2 *__restrict__ coef_i, int64_t total, int64_t last_row, int V, float inv_v,
+    double inv_v_d, float scale, const float *__restrict__ device_factor) {
   const float factor = device_factor ? *device_factor : 1.f;
   if (!FLS) scale *= factor;
   constexpr int kPerBlock = kHalfGradUnroll * kBlock * kHalfWide;  // elements per workgroup
@@ -361,40 +383,53 @@ __global__ __launch_bounds__(kBlock) void grad_flat_half_kernel(
   }
   const int rem_base = (int)(base - row_base * V);
   const int64_t wide_end = total - total % kHalfWide;  // whole 16-byte accesses end here
-  float x[kHalfGradUnroll][kHalfWide];
+  const unsigned span_bytes =
+      (unsigned)max((int64_t)0, min((int64_t)kPerBlock, wide_end - base)) * 2u;
+  const __amdgpu_buffer_rsrc_t in_buf = make_buffer((FLS ? grad : logits) + base, span_bytes);
+  const __amdgpu_buffer_rsrc_t out_buf = make_buffer(grad + base, span_bytes);
+
+  u32x4 raw[kHalfGradUnroll];
+  int rows[kHalfGradUnroll], col0[kHalfGradUnroll];
 #pragma unroll
   for (int k = 0; k < kHalfGradUnroll; ++k) {
-    const int64_t elem = base + (int64_t)(k * kBlock + (int)threadIdx.x) * kHalfWide;
-    if (!FLS && elem < wide_end) HalfIO<E, kHalfWide>::load(logits + elem, x[k]);
+    const int local = (k * kBlock + (int)threadIdx.x) * kHalfWide;
+    if (!FLS) raw[k] = __builtin_amdgcn_raw_buffer_load_b128(in_buf, (unsigned)local * 2u, 0, kAuxStream);
+    // row and column of the access's first element: idx < V + kPerBlock is exact in
+    // float, one correction step fixes the quotient
+    const int idx = rem_base + local;
+    int q = (int)((float)idx * inv_v);
+    if (q * V > idx) --q; else if ((q + 1) * V <= idx) ++q;
+    rows[k] = q;
+    col0[k] = idx - q * V;
+  }
+  float4 f0[kHalfGradUnroll], f1[kHalfGradUnroll];
+  int2 c0[kHalfGradUnroll], c1[kHalfGradUnroll];
+#pragma unroll
+  for (int k = 0; k < kHalfGradUnroll; ++k) {
+    const int64_t row0 = min(row_base + rows[k], last_row);
+    f0[k] = coef_f[row0];
+    c0[k] = coef_i[row0];
+    if (S < kHalfWide) {
+      const int64_t row1 = min(row0 + 1, last_row);
+      f1[k] = coef_f[row1];
+      c1[k] = coef_i[row1];
+    }
   }
 #pragma unroll
   for (int k = 0; k < kHalfGradUnroll; ++k) {
     const int local = (k * kBlock + (int)threadIdx.x) * kHalfWide;
-    const int64_t elem = base + local;
-    if (elem >= wide_end) break;
-    float y[kHalfWide];
-    // row and column of the access's first element: idx < V + kPerBlock is exact in
-    // float, one correction step fixes the quotient; later pieces step to the next row
-    // when the column runs past V (S divides V: at most once per piece)
-    const int idx = rem_base + local;
-    int q = (int)((float)idx * inv_v);
-    if (q * V > idx) --q; else if ((q + 1) * V <= idx) ++q;
-    int col = idx - q * V;
-    int64_t row = row_base + q;
-    float4 f = coef_f[row];
-    int2 ci = coef_i[row];
+    float x[kHalfWide], y[kHalfWide];
+    if (!FLS) unpack8<E>(raw[k], x);
 #pragma unroll
     for (int j = 0; j < kHalfWide; j += S) {
-      if (col >= V) {
-        col -= V;
-        ++row;
-        f = coef_f[row];
-        ci = coef_i[row];
-      }
-      grad_piece<S, FLS>(&x[k][j], &y[j], f, ci, col, scale, factor);
-      col += S;
+      const int cj = col0[k] + j;
+      const bool second = S < kHalfWide && cj >= V;  // S divides V: a piece never straddles
+      const float4 f = second ? f1[k] : f0[k];
+      const int2 ci = second ? c1[k] : c0[k];
+      grad_piece<S, FLS>(&x[j], &y[j], f, ci, second ? cj - V : cj, scale, factor);
     }
-    HalfIO<E, kHalfWide>::store(grad + elem, y);
+    __builtin_amdgcn_raw_buffer_store_b128(pack8<E>(y), out_buf, (unsigned)local * 2u, 0,
+                                           kAuxStreamStore);
   }
   // the last total % 8 elements (a multiple of S), S at a time
   if (S < kHalfWide && blockIdx.x == gridDim.x - 1) {
@@ -540,13 +575,13 @@ static int launch_gradient(const unsigned short *logits, const void *row_scratch
   const uintptr_t bits = reinterpret_cast<uintptr_t>(grad) |
                          (from_log_softmax ? 0 : reinterpret_cast<uintptr_t>(logits));
   const int64_t total = rows * (int64_t)V;
-  if ((bits & 15) == 0 && V < (1 << 23)) {
+  if ((bits & 15) == 0 && V >= kHalfWide && V < (1 << 23)) {
     const int64_t per_block = (int64_t)kHalfGradUnroll * kBlock * kHalfWide;
     const int64_t blocks = (total + per_block - 1) / per_block;
     if (blocks > INT32_MAX) return OT_E_BAD_ARG;
 #define OT_LAUNCH_GRADH(S_, FLS_)                                                               \
   hipLaunchKernelGGL((grad_flat_half_kernel<E, S_, FLS_>), dim3((unsigned)blocks), dim3(kBlock), \
-                     0, s, logits, grad, coef_f, coef_i, total, V, 1.0f / (float)V,             \
+                     0, s, logits, grad, coef_f, coef_i, total, rows - 1, V, 1.0f / (float)V,   \
                      1.0 / (double)V, grad_scale, device_factor)
 #define OT_LAUNCH_GRADH_S(FLS_)                        \
   switch (S) {                                         \
