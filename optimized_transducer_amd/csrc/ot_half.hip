@@ -6,11 +6,13 @@
 // 2-byte logits directly halves the traffic of both streaming passes.  Every
 // per-row quantity (denominators, log-probabilities, alpha, beta, the gradient
 // coefficients) stays float32 and goes through the float32 kernels; only
-//   lse_gather_half_kernel   per-row log-sum-exp + blank/target gather
+//   lse_gather_half_*_kernel per-row log-sum-exp + blank/target gather (flat: rows
+//                            as one stream re-shaped through LDS, for V a multiple
+//                            of 4 up to 1024; wide: aligned 16-byte pieces with
+//                            masked row ends; plain: any alignment and length)
 //   gather_half_kernel       gather only (log-softmax input)
 //   grad_flat_half_kernel    (rows, V) gradient pass, in place for logits input
-// are specific to the element type.  Rows start at multiples of V elements, so
-// the access width is the largest of 8, 4, 2, 1 elements that divides V.
+// are specific to the element type.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -182,6 +184,116 @@ __global__ __launch_bounds__(kBlock) void lse_gather_half_wide_kernel(
   }
   finish_rows<E>(dvec, lane, row_first, row_end, logits, targets, target_lengths, row_splits, N,
                  targets_cols, V, blank, den, lp);
+}
+
+// V a multiple of 4 and at most 4 * 32 * 8 elements, array 16-byte aligned: the
+// layout of the float32 denominator kernel.  A group of L lanes reduces one row (K
+// 8-byte vectors per lane), a wave G = 64 / L rows per pass.  The G rows of a pass
+// are contiguous, so the wave reads them as one flat span (lane i takes 16-byte units
+// i, i + 64, ...: every load instruction covers an aligned, contiguous 1 KiB) and
+// re-shapes the span into the row-group layout through a wave-private LDS buffer;
+// the span of the next pass is in flight while the current one is reduced.  The
+// blank/target gather reads LDS, and the workgroup's results leave in two contiguous
+// pieces at the end.
+template <class E, int L, int K>
+__global__ __launch_bounds__(kBlock) void lse_gather_half_flat_kernel(
+    const unsigned short *__restrict__ logits, const int32_t *__restrict__ targets,
+    const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits, int N,
+    int targets_cols, int64_t rows, int V, int blank, int rows_per_block, float *__restrict__ den,
+    float *__restrict__ lp) {
+  constexpr int G = kWave / L;
+  constexpr int KS = K / 2;  // 16-byte units per lane and span
+  static_assert(G >= 2 && K >= 2 && K % 2 == 0, "span of whole 16-byte units");
+  constexpr int kStageBytes = kWave * KS * 16;  // = G * L * K 8-byte vectors
+  __shared__ BlockUtterances bu;
+  __shared__ __attribute__((aligned(16))) unsigned char s_stage[kWavesPerBlock * kStageBytes];
+  __shared__ float s_den[kMaxRowsPerBlock], s_lp[2 * kMaxRowsPerBlock];
+  const int64_t row_first = (int64_t)blockIdx.x * rows_per_block;
+  const int64_t row_end = min(rows, row_first + rows_per_block);
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int sub = lane % L, g = lane / L;
+  const int nvec = V / 4;
+  unsigned char *stage = s_stage + wave * kStageBytes;
+
+  // the workgroup's rows are one raw buffer: the tail of the last span (rows past
+  // row_end) reads as zeros without a bounds branch
+  const __amdgpu_buffer_rsrc_t block_buf =
+      make_buffer(logits + row_first * (int64_t)V, (unsigned)((row_end - row_first) * V * 2));
+  u32x4 a[KS];
+  auto issue_span = [&](int64_t base) {
+    const unsigned off0 = (unsigned)(base - row_first) * (unsigned)V * 2u;
+#pragma unroll
+    for (int k = 0; k < KS; ++k)
+      a[k] = __builtin_amdgcn_raw_buffer_load_b128(block_buf, off0 + (unsigned)(k * kWave + lane) * 16u,
+                                                   0, kAuxStream);
+  };
+
+  int64_t base = row_first + (int64_t)wave * G;
+  if (base < row_end) issue_span(base);
+  // the utterance table is only needed for the gather at the end of a pass: its
+  // searches run while the first span is in flight
+  bu.load(row_splits, N, row_first, row_end - 1);
+  const int64_t lattice_rows = row_splits[N];
+
+  for (; base < row_end; base += kWavesPerBlock * G) {
+    const int64_t row = base + g;
+    const bool active = row < row_end;
+#pragma unroll
+    for (int k = 0; k < KS; ++k)
+      *reinterpret_cast<u32x4 *>(stage + (k * kWave + lane) * 16) = a[k];
+    issue_span(base + kWavesPerBlock * G);  // past row_end: all zeros, never used
+    float x[K][4];
+    float cm = OT_NEG_INF;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int j = k * L + sub;
+      // always inside the wave's buffer; slots past the row are masked
+      const uint2 r = *reinterpret_cast<const uint2 *>(stage + (g * nvec + j) * 8);
+      const bool keep = (j < nvec) & active;
+      x[k][0] = to_float<E>((unsigned short)(r.x & 0xffffu));
+      x[k][1] = to_float<E>((unsigned short)(r.x >> 16));
+      x[k][2] = to_float<E>((unsigned short)(r.y & 0xffffu));
+      x[k][3] = to_float<E>((unsigned short)(r.y >> 16));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x[k][e] = keep ? x[k][e] : OT_NEG_INF;
+        cm = fmaxf(cm, x[k][e]);
+      }
+    }
+    float m = group_allreduce<L>(cm, MaxOp());
+    if (__builtin_isinf(m)) m = 0.f;  // as ATen's logsumexp does for an all -inf / +inf row
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc += exp_fast(x[k][e] - m);
+    const float d = logf(group_allreduce<L>(acc, SumOp())) + m;
+
+    if (active) {
+      const int local = (int)(row - row_first);
+      if (sub == 0) s_den[local] = d;
+      if (sub < 2 && row < lattice_rows) {
+        const Cell c = decode_row(bu, row, nullptr, target_lengths);
+        int col = blank;
+        bool ok = true;
+        if (sub == 1) {
+          ok = c.u >= 0 && c.u < c.U && c.u < targets_cols;
+          if (ok) {
+            col = targets[(int64_t)c.b * targets_cols + c.u];
+            ok = (unsigned)col < (unsigned)V;
+          }
+        }
+        float v = 0.f;
+        if (ok) v = to_float<E>(reinterpret_cast<const unsigned short *>(stage)[g * V + col]);
+        s_lp[2 * local + sub] = ok ? v - d : OT_NEG_INF;
+      }
+    }
+  }
+  __syncthreads();
+  const int nrows = (int)(row_end - row_first);
+  const int nlp = 2 * (int)max((int64_t)0, min((int64_t)nrows, lattice_rows - row_first));
+  for (int i = threadIdx.x; i < nrows; i += kBlock) den[row_first + i] = s_den[i];
+  for (int i = threadIdx.x; i < nlp; i += kBlock) lp[2 * row_first + i] = s_lp[i];
 }
 
 // A group of L lanes reduces one row (L * kHalfK * VEC >= V), so a wave reduces
@@ -507,6 +619,40 @@ static int launch_log_probs(const unsigned short *logits, const int32_t *targets
     hipLaunchKernelGGL(gather_half_kernel<E>, dim3(blocks), dim3(kBlock), 0, s, logits, targets,
                        target_lengths, row_splits, N, targets_cols, rows, V, blank, lp);
     return launch_status();
+  }
+  if ((reinterpret_cast<uintptr_t>(logits) & 15) == 0 && V % 4 == 0) {
+    // rows as one flat stream, re-shaped through LDS
+    const int nvec = V / 4;
+    int L = 8;
+    while (L < 32 && L * 8 < nvec) L *= 2;
+    int K = 2;
+    while (K < 8 && L * K < nvec) K *= 2;
+    if (L * K >= nvec) {
+      // about 256 KiB of logits per workgroup, a whole number of wave passes
+      const int pass = kWavesPerBlock * (kWave / L);
+      int rpb = (int)((256 * 1024 / ((int64_t)V * 2)) / pass * pass);
+      if (rpb < pass) rpb = pass;
+      if (rpb > kMaxRowsPerBlock) rpb = kMaxRowsPerBlock;
+      const unsigned nblocks = (unsigned)((rows + rpb - 1) / rpb);
+#define OT_LAUNCH_LSEF(L_, K_)                                                                    \
+  hipLaunchKernelGGL((lse_gather_half_flat_kernel<E, L_, K_>), dim3(nblocks), dim3(kBlock), 0, s, \
+                     logits, targets, target_lengths, row_splits, N, targets_cols, rows, V, blank, \
+                     rpb, den, lp)
+#define OT_LAUNCH_LSEF_K(L_)                 \
+  switch (K) {                               \
+    case 2: OT_LAUNCH_LSEF(L_, 2); break;    \
+    case 4: OT_LAUNCH_LSEF(L_, 4); break;    \
+    default: OT_LAUNCH_LSEF(L_, 8); break;   \
+  }
+      switch (L) {
+        case 8: OT_LAUNCH_LSEF_K(8) break;
+        case 16: OT_LAUNCH_LSEF_K(16) break;
+        default: OT_LAUNCH_LSEF_K(32) break;
+      }
+#undef OT_LAUNCH_LSEF_K
+#undef OT_LAUNCH_LSEF
+      return launch_status();
+    }
   }
   const int64_t rows_per_block = (int64_t)kWavesPerBlock * kHalfRowsPerWave;
   const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);

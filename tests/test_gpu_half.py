@@ -33,9 +33,10 @@ def _half_batch(rng, N, tmax, umax, V, dtype, device, osf=False, scale=1.0):
     return T, U, tg, xh.to(device), xh.float().numpy()    # and their exact float32 values
 
 
-# V: 500 -> 4 elements per access, 512 -> 8, 6 -> 2, 37 -> 1; 2048 / 5000 -> 4 chunks / any length
+# V: 500 -> 4 elements per access, 512 -> 8, 6 -> 2, 37 -> 1; 2048 / 5000 -> 4 chunks / any length;
+# 8, 100, 1024: the other lane groupings of the flat denominator kernel
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f16", "bf16"])
-@pytest.mark.parametrize("V", [500, 512, 6, 37, 2048, 5000, 1030])
+@pytest.mark.parametrize("V", [500, 512, 6, 37, 2048, 5000, 1030, 8, 100, 1024])
 def test_log_probs_and_gradient_kernels(V, dtype, device):
     rng = np.random.default_rng(V)
     T, U, tg, xh, x32 = _half_batch(rng, 5, 12, 6, V, dtype, device, scale=2.0)
