@@ -303,6 +303,37 @@ int ot_gradient_apply_half(const void *logits, int32_t dtype,
 int ot_scale_by_device_scalar_half(void *x, int32_t dtype, int64_t n,
                                    const float *factor, void *stream);
 
+/* ---- output projection of the joiner fused with the denominators (no
+ * counterpart in the reference: its caller computes
+ * logits = Linear(tanh(enc + dec)) with torch, README.md:166-177, and the loss
+ * re-reads all of them for logits.logsumexp(1), cuda.cu:427) ----
+ *
+ * logits[r, v] = sum_k x[r, k] * weight[v, k] + bias[v] on the matrix cores,
+ * float32 accumulation, rounded once to `logits_dtype`, and
+ * den[r] = log sum_v exp(logits[r, v]) of exactly the stored values, taken from
+ * the accumulators: the loss then needs no pass of its own over the logits for
+ * the denominators (ot_log_probs_given_den instead of ot_log_probs).
+ *
+ * x (rows, D) and weight (V, D) row-major of `dtype` (OT_DTYPE_F16 or
+ * OT_DTYPE_BF16), 16-byte aligned, D a multiple of 32; bias (V) float32 or
+ * NULL; logits (rows, V) of logits_dtype = OT_DTYPE_F32 or `dtype`;
+ * den (rows) float32. */
+int ot_joiner_project(const void *x, const void *weight, const float *bias,
+                      int32_t dtype, int64_t rows, int32_t D, int32_t V,
+                      void *logits, int32_t logits_dtype, float *den,
+                      void *stream);
+
+/* The gather step of ot_log_probs for denominators that are already known
+ * (ComputeLogProbs, cpu.cc:52-100, without the log-sum-exp in front of it):
+ * lp[row] = (logits[row, blank], logits[row, target(row)]) - den[row];
+ * logits of `dtype` (any of the three), rows >= row_splits[N] are left alone. */
+int ot_log_probs_given_den(const void *logits, int32_t dtype, const float *den,
+                           const int32_t *targets,
+                           const int32_t *target_lengths,
+                           const int32_t *row_splits, int32_t N,
+                           int32_t targets_cols, int64_t rows, int32_t V,
+                           int32_t blank, float *lp, void *stream);
+
 /* Plain device-to-device copy kernel of n floats; used to calibrate profiler
  * byte counters against a transfer of known size. */
 int ot_copy_floats(const float *src, float *dst, int64_t n, void *stream);

@@ -34,7 +34,7 @@ def _run(cmd):
 
 
 def build_kernels():
-    srcs = [os.path.join(CSRC, f) for f in ("ot_kernels.hip", "ot_joiner.hip", "ot_half.hip")]
+    srcs = [os.path.join(CSRC, f) for f in ("ot_kernels.hip", "ot_joiner.hip", "ot_half.hip", "ot_project.hip")]
     _run([os.path.join(ROCM, "bin", "hipcc")] + HIPCC_FLAGS +
          ["-I", INCLUDE, "-I", CSRC] + srcs + ["-o", KERNEL_LIB])
     return KERNEL_LIB

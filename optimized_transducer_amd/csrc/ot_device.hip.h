@@ -265,5 +265,24 @@ template <> struct Vec<1> {
   __device__ __forceinline__ void store_lds(float *p) const { *p = v[0]; }
 };
 
+// element types of 2-byte arrays, and their conversions
+struct F16 {};   // IEEE binary16
+struct BF16 {};  // bfloat16: the upper half of a float32
+
+template <class E> __device__ __forceinline__ float to_float(unsigned short bits);
+template <> __device__ __forceinline__ float to_float<F16>(unsigned short bits) {
+  return (float)__builtin_bit_cast(_Float16, bits);
+}
+template <> __device__ __forceinline__ float to_float<BF16>(unsigned short bits) {
+  return __builtin_bit_cast(float, (unsigned)bits << 16);
+}
+template <class E> __device__ __forceinline__ unsigned short from_float(float x);
+template <> __device__ __forceinline__ unsigned short from_float<F16>(float x) {
+  return __builtin_bit_cast(unsigned short, (_Float16)x);  // round to nearest even
+}
+template <> __device__ __forceinline__ unsigned short from_float<BF16>(float x) {
+  return __builtin_bit_cast(unsigned short, (__bf16)x);  // round to nearest even
+}
+
 }  // namespace ot
 #endif  // OT_DEVICE_HIP_H_

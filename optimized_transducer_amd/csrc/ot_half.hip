@@ -21,24 +21,6 @@
 
 namespace ot {
 
-struct F16 {};   // IEEE binary16
-struct BF16 {};  // bfloat16: the upper half of a float32
-
-template <class E> __device__ __forceinline__ float to_float(unsigned short bits);
-template <> __device__ __forceinline__ float to_float<F16>(unsigned short bits) {
-  return (float)__builtin_bit_cast(_Float16, bits);
-}
-template <> __device__ __forceinline__ float to_float<BF16>(unsigned short bits) {
-  return __builtin_bit_cast(float, (unsigned)bits << 16);
-}
-template <class E> __device__ __forceinline__ unsigned short from_float(float x);
-template <> __device__ __forceinline__ unsigned short from_float<F16>(float x) {
-  return __builtin_bit_cast(unsigned short, (_Float16)x);  // round to nearest even
-}
-template <> __device__ __forceinline__ unsigned short from_float<BF16>(float x) {
-  return __builtin_bit_cast(unsigned short, (__bf16)x);  // round to nearest even
-}
-
 // VEC consecutive elements <-> floats; VEC * 2 bytes per access
 template <class E, int VEC> struct HalfIO {
   static_assert(VEC == 1 || VEC == 2 || VEC == 4 || VEC == 8, "elements per access");

@@ -224,3 +224,21 @@ def pack_joiner_backward(grad_out, encoder_out, decoder_out, logit_lengths, targ
         gd[i, :U1] = gi.sum(0)
         r += T * U1
     return ge, gd, ae, ad
+
+
+# ---------------------------------------------------------------- joiner output projection
+def project_joiner(x, weight, bias=None):
+    """The caller-side projection in front of the loss (README.md:176-177,
+    `logits = linear(activation(x))`): x @ weight.T + bias in float64, and the
+    sum of the absolute values of the terms of every entry (the scale of the rounding
+    error of a float32 accumulation in any order).  The per-row denominators of the
+    result are log_sum_exp's, as for any logits (cpu.cc:770)."""
+    x = np.asarray(x, dtype=np.float64)
+    w = np.asarray(weight, dtype=np.float64)
+    out = x @ w.T
+    mag = np.abs(x) @ np.abs(w).T
+    if bias is not None:
+        b = np.asarray(bias, dtype=np.float64)
+        out = out + b[None, :]
+        mag = mag + np.abs(b)[None, :]
+    return out, mag

@@ -223,3 +223,31 @@ def gradient_half(logits, lp, den, alpha, beta, targets, T, U, splits, blank, fr
         ctypes.c_int32(V), ctypes.c_int32(int(from_log_softmax)), ctypes.c_float(grad_scale),
         ptr(device_factor), ptr(grad), stream()))
     return grad
+
+
+ANY_DTYPE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def joiner_project(x, weight, bias, out_dtype, logits=None):
+    rows, D = x.shape
+    V = weight.shape[0]
+    if logits is None:
+        logits = torch.full((rows, V), float("nan"), dtype=out_dtype, device=x.device)
+    den = torch.full((rows,), float("nan"), dtype=torch.float32, device=x.device)
+    check(lib().ot_joiner_project(ptr(x), ptr(weight), ptr(bias), ctypes.c_int32(DTYPE[x.dtype]),
+                                  ctypes.c_int64(rows), ctypes.c_int32(D), ctypes.c_int32(V),
+                                  ptr(logits), ctypes.c_int32(ANY_DTYPE[out_dtype]), ptr(den),
+                                  stream()))
+    return logits, den
+
+
+def log_probs_given_den(logits, den, targets, U, splits, blank):
+    rows, V = logits.shape
+    lp = torch.full((rows, 2), float("nan"), dtype=torch.float32, device=logits.device)
+    cols = targets.shape[1]
+    check(lib().ot_log_probs_given_den(ptr(logits), ctypes.c_int32(ANY_DTYPE[logits.dtype]), ptr(den),
+                                       ptr(targets if cols else None), ptr(U), ptr(splits),
+                                       ctypes.c_int32(U.numel()), ctypes.c_int32(cols),
+                                       ctypes.c_int64(rows), ctypes.c_int32(V), ctypes.c_int32(blank),
+                                       ptr(lp), stream()))
+    return lp

@@ -1,0 +1,91 @@
+"""Output projection of the joiner fused with the denominators (an addition to the
+reference, whose caller runs torch's Linear and whose loss then re-reads the logits
+for logsumexp, README.md:176-177, cuda.cu:427).
+
+The oracle forms x @ W.T + bias in float64 from the 2-byte inputs (exact in float64)
+and gives the scale of a float32 accumulation's rounding error; logits stored in a
+2-byte type may in addition be off by one rounding of that type.  The denominators
+are checked against the log-sum-exp of the values the kernel itself stored, which is
+what the loss's own denominator pass would compute from them."""
+import numpy as np
+import pytest
+import torch
+
+import cabi
+import helpers
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+HALF = {"f16": torch.float16, "bf16": torch.bfloat16}
+ULP = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8, torch.float32: 0.0}
+
+
+def _inputs(rng, rows, D, V, dtype, device, bias=True, scale=1.0):
+    x = torch.from_numpy(np.tanh(rng.standard_normal((rows, D))).astype(np.float32)).to(dtype)
+    w = torch.from_numpy((rng.standard_normal((V, D)) * scale / np.sqrt(D)).astype(np.float32)).to(dtype)
+    b = torch.from_numpy(rng.standard_normal(V).astype(np.float32)) if bias else None
+    return x.to(device), w.to(device), None if b is None else b.to(device)
+
+
+def _check(x, w, b, out_dtype):
+    logits, den = cabi.joiner_project(x, w, b, out_dtype)
+    want, mag = oracle.project_joiner(x.float().cpu().numpy(), w.float().cpu().numpy(),
+                                      None if b is None else b.cpu().numpy())
+    got = logits.float().cpu().numpy().astype(np.float64)
+    assert not np.isnan(got).any()
+    tol = 2e-6 * mag + ULP[out_dtype] * np.abs(want) * 1.001 + 1e-30
+    assert (np.abs(got - want) <= tol).all(), (np.abs(got - want) / tol).max()
+    # denominators of the stored values
+    m = got.max(1)
+    ref = m + np.log(np.exp(got - m[:, None]).sum(1))
+    d = den.cpu().numpy().astype(np.float64)
+    assert (np.abs(d - ref) <= 4e-7 * np.maximum(np.abs(ref), np.abs(m)) + 1e-6).all(), np.abs(d - ref).max()
+    return logits, den
+
+
+@pytest.mark.parametrize("out", ["f32", "same"])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("rows,D,V", [(700, 64, 500), (256, 32, 128), (1, 512, 37), (513, 96, 1030),
+                                      (300, 128, 6), (64, 256, 130)])
+def test_projection_and_denominators(rows, D, V, dtype, out, device):
+    rng = np.random.default_rng(rows * 7 + V)
+    dt = HALF[dtype]
+    x, w, b = _inputs(rng, rows, D, V, dt, device)
+    _check(x, w, b, torch.float32 if out == "f32" else dt)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_no_bias_and_large_values(dtype, device):
+    rng = np.random.default_rng(5)
+    dt = HALF[dtype]
+    x, w, _ = _inputs(rng, 200, 64, 300, dt, device, bias=False, scale=40.0)
+    _check(x, w, None, torch.float32)
+    _check(x, w, None, dt)
+
+
+def test_masked_logits_through_the_bias(device):
+    # a -inf bias masks vocabulary entries: they must drop out of the denominator
+    rng = np.random.default_rng(9)
+    x, w, b = _inputs(rng, 100, 64, 200, torch.bfloat16, device)
+    b[50:120] = -float("inf")
+    logits, den = cabi.joiner_project(x, w, b, torch.float32)
+    got = logits.cpu().numpy().astype(np.float64)
+    assert np.isneginf(got[:, 50:120]).all() and np.isfinite(got[:, :50]).all()
+    ref = torch.logsumexp(logits.double(), 1).cpu().numpy()
+    assert np.allclose(den.cpu().numpy(), ref, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_log_probs_given_denominators(dtype, device):
+    rng = np.random.default_rng(3)
+    T, U, tg, x = helpers.random_batch(rng, 5, 9, 6, 41)
+    xd = torch.from_numpy(x).to(dtype).to(device)
+    x32 = xd.float().cpu().numpy()
+    dT, dU, dtg = (torch.from_numpy(a).to(device) for a in (T, U, tg))
+    splits, _ = cabi.row_splits(dT, dU, dtg)
+    den = oracle.logsumexp(x32)
+    want = oracle.log_probs(x32, den, tg, T, U, 0)
+    got = cabi.log_probs_given_den(xd, torch.from_numpy(den).to(device), dtg, dU, splits, 0).cpu().numpy()
+    m = np.isfinite(want)
+    assert (got[m] == want[m]).all() and np.isneginf(got[~m]).all()
