@@ -26,7 +26,8 @@ if _torch.__version__.split("+")[0] != _built.split("+")[0]:
     )
 
 from .transducer_loss import TransducerLoss, TransducerLossFunction, transducer_loss  # noqa: E402,F401
-from .joiner import PackJoinerFunction, pack_joiner  # noqa: E402,F401
+from .joiner import (PackJoinerFunction, ProjectJoinerFunction, pack_joiner,  # noqa: E402,F401
+                     project_joiner)
 
 __all__ = ["TransducerLoss", "TransducerLossFunction", "transducer_loss", "PackJoinerFunction",
-           "pack_joiner"]
+           "pack_joiner", "ProjectJoinerFunction", "project_joiner"]

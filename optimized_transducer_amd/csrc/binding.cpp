@@ -146,14 +146,18 @@ inline int half_dtype(const torch::Tensor &t) {
   return OT_DTYPE_F32;
 }
 
+// With `denominators` given (the per-row log-sum-exp of logits input, as
+// joiner_project produces them), the pass over the logits for them is skipped.
 // With `coefficients` set, the (rows, V) gradient pass is left to
 // apply_deferred_gradient: the per-row coefficients go into a tensor of their own,
 // handed back through the pointer, and the returned gradient is None.
 std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
     torch::Tensor &logits, const torch::Tensor &targets, const torch::Tensor &logit_lengths,
     const torch::Tensor &target_lengths, int32_t blank, bool from_log_softmax,
-    bool one_sym_per_frame, double grad_scale, torch::Tensor *coefficients) {
+    bool one_sym_per_frame, double grad_scale, torch::Tensor *coefficients,
+    const torch::optional<torch::Tensor> &denominators = torch::nullopt) {
   const bool defer = coefficients != nullptr;
+  const bool have_den = denominators.has_value() && denominators->defined();
   auto logits_arg = torch::TensorArg(logits, "logits", 0);
   auto targets_arg = torch::TensorArg(targets, "targets", 1);
   auto logit_lengths_arg = torch::TensorArg(logit_lengths, "logit_lengths", 2);
@@ -206,6 +210,14 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   TORCH_CHECK(rows > 0 && V > 0, "logits must not be empty");
   TORCH_CHECK(rows <= INT32_MAX && N < INT32_MAX && V <= INT32_MAX && S < OT_MAX_U1 * 64,
               "tensor sizes exceed what 32-bit row offsets can address");
+  if (have_den) {
+    TORCH_CHECK(!from_log_softmax, "denominators belong to logits input (from_log_softmax=False)");
+    TORCH_CHECK(denominators->scalar_type() == torch::kFloat && denominators->dim() == 1 &&
+                    denominators->size(0) == rows && denominators->is_contiguous() &&
+                    denominators->device() == logits.device(),
+                "denominators must be a contiguous float32 tensor of shape (logits.size(0),) on "
+                "the device of logits");
+  }
 
   c10::hip::HIPGuardMasqueradingAsCUDA device_guard(logits.device());
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
@@ -230,7 +242,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   }
   auto *row_splits = reinterpret_cast<int32_t *>(w);
   auto *scores_beta = reinterpret_cast<float *>(w + off_sbeta);
-  auto *den = reinterpret_cast<float *>(w + off_den);
+  auto *den = have_den ? denominators->data_ptr<float>() : reinterpret_cast<float *>(w + off_den);
   auto *lp = reinterpret_cast<float *>(w + off_lp);
   auto *alpha = reinterpret_cast<float *>(w + off_alpha);
   auto *beta = reinterpret_cast<float *>(w + off_beta);
@@ -268,7 +280,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   //   main:  lse[rows < h]  lse[rows >= h]        grad[part A]      grad[part B]
   //   side:                 lattice+coeff[A]      lattice+coeff[B]
   // h is a row count, part A = the utterances that end at or before row h.
-  const bool overlap = overlap_enabled() && dtype == OT_DTYPE_F32 && N >= 2 &&
+  const bool overlap = overlap_enabled() && dtype == OT_DTYPE_F32 && !have_den && N >= 2 &&
                        rows * V >= kOverlapMinElements;
   const int64_t half = overlap ? rows / 2 : rows;
   EventGuard lse_a_done, lse_b_done;
@@ -277,8 +289,12 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   // from device data, so it can run while the host waits for the facts.
   const bool blank_ok = (0 <= blank && blank < V);
   if (blank_ok) {
-    ScopedTimer timer(from_log_softmax ? "gather" : "lse_gather", stream);
-    if (dtype != OT_DTYPE_F32) {
+    ScopedTimer timer(from_log_softmax ? "gather" : have_den ? "gather_given_den" : "lse_gather",
+                      stream);
+    if (have_den) {
+      OT_CHECK(ot_log_probs_given_den(p_logits, dtype, den, p_targets, p_U, row_splits, (int32_t)N,
+                                      (int32_t)S, rows, (int32_t)V, blank, lp, stream));
+    } else if (dtype != OT_DTYPE_F32) {
       OT_CHECK(ot_log_probs_half(p_logits, dtype, p_targets, p_U, row_splits, (int32_t)N,
                                  (int32_t)S, rows, (int32_t)V, blank, from_log_softmax, den, lp,
                                  stream));
@@ -397,9 +413,10 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_transducer_loss
 std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_transducer_loss_scaled(
     torch::Tensor &logits, const torch::Tensor &targets, const torch::Tensor &logit_lengths,
     const torch::Tensor &target_lengths, int32_t blank, bool from_log_softmax,
-    bool one_sym_per_frame, double grad_scale) {
+    bool one_sym_per_frame, double grad_scale,
+    const torch::optional<torch::Tensor> &denominators) {
   return compute_impl(logits, targets, logit_lengths, target_lengths, blank, from_log_softmax,
-                      one_sym_per_frame, grad_scale, nullptr);
+                      one_sym_per_frame, grad_scale, nullptr, denominators);
 }
 
 // Forward half of the deferred mode: everything but the (rows, V) pass.  Returns
@@ -408,10 +425,11 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_transducer_loss
 std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_transducer_loss_deferred(
     torch::Tensor &logits, const torch::Tensor &targets, const torch::Tensor &logit_lengths,
     const torch::Tensor &target_lengths, int32_t blank, bool from_log_softmax,
-    bool one_sym_per_frame, double grad_scale) {
+    bool one_sym_per_frame, double grad_scale,
+    const torch::optional<torch::Tensor> &denominators) {
   torch::Tensor coefficients;
   auto out = compute_impl(logits, targets, logit_lengths, target_lengths, blank, from_log_softmax,
-                          one_sym_per_frame, grad_scale, &coefficients);
+                          one_sym_per_frame, grad_scale, &coefficients, denominators);
   if (coefficients.defined()) return {out.first, coefficients};
   return {out.first, torch::nullopt};
 }
@@ -615,6 +633,43 @@ std::pair<torch::Tensor, torch::Tensor> joiner_unpack_grad(
 
 }  // namespace
 
+// Output projection of the joiner with the denominators of the loss from the
+// accumulators (ot_joiner_project): logits (rows, V) float32 or of x's dtype, den (rows).
+std::pair<torch::Tensor, torch::Tensor> joiner_project(const torch::Tensor &x,
+                                                       const torch::Tensor &weight,
+                                                       const torch::optional<torch::Tensor> &bias,
+                                                       bool float32_logits) {
+  const int dtype = half_dtype(x);
+  TORCH_CHECK(dtype != OT_DTYPE_F32, "joiner_project takes float16 or bfloat16 x, got ", x.scalar_type());
+  TORCH_CHECK(x.is_cuda() && weight.device() == x.device(), "x and weight must be on one HIP device");
+  TORCH_CHECK(x.dim() == 2 && weight.dim() == 2 && x.size(1) == weight.size(1) &&
+                  weight.scalar_type() == x.scalar_type() && x.is_contiguous() && weight.is_contiguous(),
+              "expect contiguous x (rows, D) and weight (V, D) of one dtype");
+  const int64_t rows = x.size(0), D = x.size(1), V = weight.size(0);
+  TORCH_CHECK(rows > 0 && V > 0 && D > 0 && D % 64 == 0 && rows <= INT32_MAX,
+              "joiner_project needs rows > 0, V > 0 and D a positive multiple of 64, got rows = ", rows,
+              ", V = ", V, ", D = ", D);
+  torch::Tensor b;
+  if (bias.has_value() && bias->defined()) {
+    TORCH_CHECK(bias->dim() == 1 && bias->size(0) == V && bias->device() == x.device(),
+                "bias must have shape (V,) on the device of x");
+    b = bias->to(torch::kFloat).contiguous();
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA device_guard(x.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+  torch::Tensor logits =
+      torch::empty({rows, V}, x.options().dtype(float32_logits ? torch::kFloat : x.scalar_type()));
+  torch::Tensor den = torch::empty({rows}, x.options().dtype(torch::kFloat));
+  {
+    ScopedTimer timer("joiner_project", stream);
+    OT_CHECK(ot_joiner_project(x.data_ptr(), weight.data_ptr(),
+                               b.defined() ? b.data_ptr<float>() : nullptr, dtype, rows, (int32_t)D,
+                               (int32_t)V, logits.data_ptr(), float32_logits ? OT_DTYPE_F32 : dtype,
+                               den.data_ptr<float>(), stream));
+  }
+  return {logits, den};
+}
+
 PYBIND11_MODULE(_optimized_transducer, m) {
   m.doc() = "MI355X-native transducer loss (drop-in for optimized_transducer's extension module)";
 #ifdef OT_BUILT_WITH_TORCH
@@ -628,11 +683,14 @@ PYBIND11_MODULE(_optimized_transducer, m) {
   m.def("compute_transducer_loss_scaled", &compute_transducer_loss_scaled, py::arg("logits"), py::arg("targets"),
         py::arg("logit_lengths"), py::arg("target_lengths"), py::arg("blank"),
         py::arg("from_log_softmax"), py::arg("one_sym_per_frame"), py::arg("grad_scale"),
+        py::arg("denominators") = py::none(),
         "Same as compute_transducer_loss with the gradient multiplied by grad_scale in the "
-        "gradient kernel (folds the `grad /= N` of reduction='mean').");
+        "gradient kernel (folds the `grad /= N` of reduction='mean'); denominators: the per-row "
+        "log-sum-exp of the logits if already known (joiner_project), else None.");
   m.def("compute_transducer_loss_deferred", &compute_transducer_loss_deferred, py::arg("logits"),
         py::arg("targets"), py::arg("logit_lengths"), py::arg("target_lengths"), py::arg("blank"),
         py::arg("from_log_softmax"), py::arg("one_sym_per_frame"), py::arg("grad_scale"),
+        py::arg("denominators") = py::none(),
         "Everything but the (rows, V) gradient pass: returns (scores, per-row coefficients or "
         "None) and leaves logits untouched.");
   m.def("apply_deferred_gradient", &apply_deferred_gradient, py::arg("logits"),
@@ -651,6 +709,10 @@ PYBIND11_MODULE(_optimized_transducer, m) {
         py::arg("decoder_out"), py::arg("logit_lengths"), py::arg("target_lengths"),
         py::arg("row_splits"), py::arg("activation"),
         "Gradient of joiner_pack: (grad_encoder_out, grad_decoder_out).");
+  m.def("joiner_project", &joiner_project, py::arg("x"), py::arg("weight"), py::arg("bias"),
+        py::arg("float32_logits"),
+        "logits = x @ weight.T + bias for float16 / bfloat16 x (rows, D) and weight (V, D) on the "
+        "matrix cores, and their per-row log-sum-exp: returns (logits, denominators).");
   m.def("set_profiling", &set_profiling, py::arg("on"));
   m.def("set_overlap", &set_overlap, py::arg("on"),
         "Run the lattice kernel of one half of a large batch on a second stream while the "

@@ -9,19 +9,21 @@
 // the loss then starts from its gather step and the logits are read once, by the
 // gradient pass, instead of twice.
 //
-// Shape of the computation.  A workgroup of 4 waves owns 256 packed rows, a wave 64
-// of them, and walks over the vocabulary in passes of 128 columns; per pass a wave
-// holds a 128 x 64 block of logits^T in 8 accumulator tiles of 32 x 32
+// Shape of the computation.  A workgroup of 8 waves owns 128 packed rows and walks
+// over the vocabulary in passes of 512 columns (one pass for V <= 512, so rows are
+// stored whole and the activations are read once); the waves form a 2 x 4 grid, a
+// wave holds a 128 x 64 block of logits^T in 8 accumulator tiles of 32 x 32
 // (v_mfma_f32_32x32x16).  The product is formed transposed (vocabulary along the
 // tile's rows, packed rows along its columns) because an accumulator lane then
 // holds 16 values of ONE packed row per tile: the running (max, sum) of the row
-// stays in that lane and its partner 32 lanes up, with no cross-lane reduction
-// until the very end.  W streams through LDS in stages of 32 k-values (shared by the
-// 4 waves, double-buffered, 16-byte slots XOR-swizzled against bank conflicts); the
-// activations go from global memory straight into the operand registers, 32
-// contiguous bytes per lane and stage.  The bias initialises the accumulators.
-// Before the store, v_permlane32_swap exchanges half of each tile between a lane
-// and its partner so that every lane owns 16 consecutive columns of its row.
+// stays in that lane, with no cross-lane reduction until the very end, where the
+// lane's partner 32 lanes up and the 4 waves of the row are merged.  W and x
+// stream through LDS in stages of 32 k-values (two buffers, 16-byte slots
+// XOR-swizzled against bank conflicts); the global loads of a stage are issued two
+// stages ahead into one of two register sets, because one stage of matrix work is
+// shorter than a trip to memory.  The bias initialises the accumulators.  The
+// stores go through a small wave-private LDS tile that turns the accumulator layout
+// into whole 128-byte pieces of rows.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -39,10 +41,18 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ unsigned as_u32(float v) { return __builtin_bit_cast(unsigned, v); }
 __device__ __forceinline__ float as_f32(unsigned v) { return __builtin_bit_cast(float, v); }
 
-constexpr int kProjRows = 256;  // packed rows per workgroup
-constexpr int kProjCols = 128;  // vocabulary columns per pass
-constexpr int kProjK = 32;      // k-values per LDS stage
-constexpr int kProjStageBytes = kProjCols * kProjK * 2;
+constexpr int kProjRows = 128;     // packed rows per workgroup (2 waves)
+constexpr int kProjCols = 256;     // vocabulary columns per pass (2 waves)
+constexpr int kProjK = 32;         // k-values per LDS stage
+constexpr int kProjThreads = 256;
+constexpr int kProjWBytes = kProjCols * kProjK * 2;
+constexpr int kProjXBytes = kProjRows * kProjK * 2;
+constexpr int kProjStageBytes = kProjWBytes + kProjXBytes;
+constexpr int kProjWPieces = kProjWBytes / 16 / kProjThreads;  // 16-byte pieces per thread: 4
+constexpr int kProjXPieces = kProjXBytes / 16 / kProjThreads;  // 2
+// store tile of a wave: 32 rows x 32 float columns, rows 9 sixteen-byte units apart
+constexpr int kProjTilePitch = 32 * 4 + 16;
+constexpr int kProjTileBytes = 32 * kProjTilePitch;
 
 template <class E>
 __device__ __forceinline__ f32x16 mfma_32x32x16(u32x4 a, u32x4 b, f32x16 c);
@@ -57,16 +67,26 @@ __device__ __forceinline__ f32x16 mfma_32x32x16<F16>(u32x4 a, u32x4 b, f32x16 c)
                                                 __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
+// one stage's worth of global data of a thread, on its way to LDS
+struct ProjStage {
+  u32x4 w[kProjWPieces];
+  u32x4 x[kProjXPieces];
+};
+
 // E: element type of x and W.  OUT_F32: logits are float32, else of type E.
 // SV: elements per store (SV * element size divides the row pitch and the base).
+// D is a multiple of 64 (an even number of stages).
 template <class E, bool OUT_F32, int SV>
-__global__ __launch_bounds__(256, 2) void joiner_project_kernel(
+__global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
     const unsigned short *__restrict__ x, const unsigned short *__restrict__ w,
     const float *__restrict__ bias, int64_t rows, int D, int V, void *__restrict__ logits,
     float *__restrict__ den) {
-  __shared__ __attribute__((aligned(16))) unsigned char s_w[2 * kProjStageBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char s_stage[2 * kProjStageBytes];
+  __shared__ float2 s_part[2][kProjRows];
+  __shared__ __attribute__((aligned(16))) unsigned char s_tile[4 * kProjTileBytes];
   constexpr unsigned kOutBytes = OUT_F32 ? 4u : 2u;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
   const int c = lane & 31, h = lane >> 5;
   const int64_t row0 = (int64_t)blockIdx.x * kProjRows;
   const unsigned nrows = (unsigned)min((int64_t)kProjRows, rows - row0);
@@ -78,57 +98,86 @@ __global__ __launch_bounds__(256, 2) void joiner_project_kernel(
   const __amdgpu_buffer_rsrc_t obuf =
       make_buffer(static_cast<char *>(logits) + row0 * V * kOutBytes, nrows * (unsigned)V * kOutBytes);
 
-  // operand addressing.  MFMA step ks of a stage: lane group h supplies k-values
-  // k0 + 16 h + 8 ks .. + 7 of both operands.
-  unsigned xoff[2];
+  // stage copy: a stage is 32 k-values = 4 chunks of 16 bytes per row; chunk cc of
+  // row r lives in slot 4 r + (cc ^ ((r >> 2) & 3)).  Thread t moves pieces
+  // t, t + 512, ... of W (piece p: row p / 4, chunk p % 4) and piece t of x.
+  // Pieces t + 256 q of a thread are 64 rows apart: same chunk, same swizzle.
+  const unsigned piece_src = ((unsigned)(tid >> 2) * (unsigned)D + 8u * (tid & 3)) * 2u;
+  const unsigned piece_dst = (unsigned)(4 * (tid >> 2) + ((tid & 3) ^ ((tid >> 4) & 3))) * 16u;
+  const unsigned piece_src_step = 64u * (unsigned)D * 2u;
+  constexpr unsigned kPieceDstStep = 64u * 4u * 16u;
+  // fragments.  MFMA step ks of a stage takes chunk 2 h + ks from lane group h of both
+  // operands: W row 128 wn + 32 vt + c, x row 64 wm + 32 rs + c
+  unsigned wfrag[2], xfrag[2];
 #pragma unroll
-  for (int rs = 0; rs < 2; ++rs)
-    xoff[rs] = ((unsigned)(64 * wave + 32 * rs + c) * (unsigned)D + 16u * h) * 2u;
-  // W stage copy: thread t moves 16-byte pieces p = t, t + 256; piece p is k-chunk p % 4
-  // of vocabulary row p / 4 and goes to slot 4 v + (chunk ^ ((v >> 1) & 3))
-  unsigned wsrc[2], wdst[2];
-#pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    const int p = tid + 256 * q, v = p >> 2, cc = p & 3;
-    wsrc[q] = ((unsigned)v * (unsigned)D + 8u * cc) * 2u;
-    wdst[q] = (unsigned)(4 * v + (cc ^ ((v >> 1) & 3))) * 16u;
+  for (int ks = 0; ks < 2; ++ks) {
+    const unsigned chunk = (unsigned)((2 * h + ks) ^ ((c >> 2) & 3));
+    wfrag[ks] = ((unsigned)(4 * (128 * wn + c)) + chunk) * 16u;
+    xfrag[ks] = kProjWBytes + ((unsigned)(4 * (64 * wm + c)) + chunk) * 16u;
   }
-  // fragment of vocabulary tile vt, step ks: row 32 vt + c, chunk 2 h + ks
-  unsigned wfrag[2];
-#pragma unroll
-  for (int ks = 0; ks < 2; ++ks) wfrag[ks] = (unsigned)(4 * c + ((2 * h + ks) ^ ((c >> 1) & 3))) * 16u;
 
   const int ksteps = D / kProjK;
-  const int ntiles = (V + kProjCols - 1) / kProjCols;
-  const int nstages = ntiles * ksteps;
+  const int npasses = (V + kProjCols - 1) / kProjCols;
 
-  u32x4 wreg[2], xreg[2][2], xnext[2][2];
-  auto load_stage = [&](int nt, int kk, u32x4 (&xr)[2][2]) {
-    const unsigned wbase = ((unsigned)(nt * kProjCols) * (unsigned)D + (unsigned)(kk * kProjK)) * 2u;
+  // global loads run two stages ahead of the matrix work
+  // Loads past the last stage are issued all the same (W reads as zeros there, x is
+  // re-read): with a branch around them the number of loads in flight would not be
+  // known at compile time and every wait would have to drain them all.
+  int load_pass = 0, load_kk = 0;
+  auto load_stage = [&](ProjStage &st) {
+    const unsigned wbase =
+        ((unsigned)(load_pass * kProjCols) * (unsigned)D + (unsigned)(load_kk * kProjK)) * 2u;
 #pragma unroll
-    for (int q = 0; q < 2; ++q) wreg[q] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, wbase + wsrc[q], 0, 0);
+    for (int q = 0; q < kProjWPieces; ++q)
+      st.w[q] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, piece_src, wbase + q * piece_src_step, 0);
 #pragma unroll
-    for (int rs = 0; rs < 2; ++rs)
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
-        xr[rs][ks] = __builtin_amdgcn_raw_buffer_load_b128(
-            xbuf, xoff[rs] + (unsigned)(kk * kProjK) * 2u + 16u * ks, 0, 0);
+    for (int q = 0; q < kProjXPieces; ++q)
+      st.x[q] = __builtin_amdgcn_raw_buffer_load_b128(
+          xbuf, piece_src, (unsigned)(load_kk * kProjK) * 2u + q * piece_src_step, 0);
+    if (++load_kk == ksteps) {
+      load_kk = 0;
+      ++load_pass;
+    }
   };
-  auto store_stage = [&](int buf) {
+  auto store_stage = [&](const ProjStage &st, int buf) {
+    unsigned char *dst = s_stage + buf * kProjStageBytes;
 #pragma unroll
-    for (int q = 0; q < 2; ++q)
-      *reinterpret_cast<u32x4 *>(s_w + buf * kProjStageBytes + wdst[q]) = wreg[q];
+    for (int q = 0; q < kProjWPieces; ++q)
+      *reinterpret_cast<u32x4 *>(dst + piece_dst + q * kPieceDstStep) = st.w[q];
+#pragma unroll
+    for (int q = 0; q < kProjXPieces; ++q)
+      *reinterpret_cast<u32x4 *>(dst + kProjWBytes + piece_dst + q * kPieceDstStep) = st.x[q];
+  };
+
+  f32x16 acc[2][4];
+  auto compute_stage = [&](int buf) {
+    const unsigned char *src = s_stage + buf * kProjStageBytes;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      u32x4 wf[4], xf[2];
+#pragma unroll
+      for (int vt = 0; vt < 4; ++vt)
+        wf[vt] = *reinterpret_cast<const u32x4 *>(src + vt * (32 * 4 * 16) + wfrag[ks]);
+#pragma unroll
+      for (int rs = 0; rs < 2; ++rs)
+        xf[rs] = *reinterpret_cast<const u32x4 *>(src + rs * (32 * 4 * 16) + xfrag[ks]);
+#pragma unroll
+      for (int vt = 0; vt < 4; ++vt)
+#pragma unroll
+        for (int rs = 0; rs < 2; ++rs) acc[rs][vt] = mfma_32x32x16<E>(wf[vt], xf[rs], acc[rs][vt]);
+    }
   };
 
   float m_run[2] = {OT_NEG_INF, OT_NEG_INF}, s_run[2] = {0.f, 0.f};
-  load_stage(0, 0, xreg);
-  store_stage(0);
-  int stage = 0;
-  for (int nt = 0; nt < ntiles; ++nt) {
-    const int n0 = nt * kProjCols;
+  ProjStage set_a, set_b;
+  load_stage(set_a);
+  load_stage(set_b);
+  store_stage(set_a, 0);
+  load_stage(set_a);
+  for (int pass = 0; pass < npasses; ++pass) {
+    const int n0 = pass * kProjCols + 128 * wn;  // first column of this wave in the pass
     // accumulators start from the bias: tile (rs, vt), register 4 j + i holds vocabulary
-    // entry n0 + 32 vt + 8 j + 4 h + i of packed row 32 rs + c
-    f32x16 acc[2][4];
+    // entry n0 + 32 vt + 8 j + 4 h + i of packed row 64 wm + 32 rs + c
 #pragma unroll
     for (int vt = 0; vt < 4; ++vt)
 #pragma unroll
@@ -142,131 +191,122 @@ __global__ __launch_bounds__(256, 2) void joiner_project_kernel(
           acc[1][vt][4 * j + i] = b4[i];
         }
       }
-    for (int kk = 0; kk < ksteps; ++kk, ++stage) {
-      const bool more = stage + 1 < nstages;
-      if (more) {
-        const bool wrap = kk + 1 == ksteps;
-        load_stage(wrap ? nt + 1 : nt, wrap ? 0 : kk + 1, xnext);
-      }
-      lds_barrier();  // this stage's W is in LDS; the other buffer is free again
-      const unsigned char *sw = s_w + (stage & 1) * kProjStageBytes;
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        u32x4 wf[4];
-#pragma unroll
-        for (int vt = 0; vt < 4; ++vt)
-          wf[vt] = *reinterpret_cast<const u32x4 *>(sw + vt * (32 * 4 * 16) + wfrag[ks]);
-#pragma unroll
-        for (int vt = 0; vt < 4; ++vt)
-#pragma unroll
-          for (int rs = 0; rs < 2; ++rs)
-            acc[rs][vt] = mfma_32x32x16<E>(wf[vt], xreg[rs][ks], acc[rs][vt]);
-      }
-      if (more) {
-        store_stage((stage + 1) & 1);
-#pragma unroll
-        for (int rs = 0; rs < 2; ++rs)
-#pragma unroll
-          for (int ks = 0; ks < 2; ++ks) xreg[rs][ks] = xnext[rs][ks];
-      }
+    for (int kk = 0; kk < ksteps; kk += 2) {
+      // even stage: buffer 0 is complete, buffer 1 is free; set_b holds the next stage
+      lds_barrier();
+      store_stage(set_b, 1);
+      load_stage(set_b);
+      compute_stage(0);
+      // odd stage
+      lds_barrier();
+      store_stage(set_a, 0);
+      load_stage(set_a);
+      compute_stage(1);
     }
 
-    // epilogue of the pass: round, update the row's running (max, sum), store
-    const bool ragged = n0 + kProjCols > V;  // the last pass may reach past V
+    // epilogue of the pass: round, update the row's running (max, sum), store.
+    // A tile's values go through a wave-private LDS tile (32 rows x 32 columns) that
+    // turns the accumulator layout (one 16-byte piece per lane and row) into whole
+    // 128-byte (64-byte for 2-byte logits) pieces of rows per store instruction.
+    const bool ragged = n0 + 128 > V;  // this wave's columns may reach past V
+    unsigned char *tile = s_tile + wave * kProjTileBytes;
+    constexpr int kTilePitch = OUT_F32 ? kProjTilePitch : kProjTilePitch / 2 + 8;  // 144 / 80 bytes
+    constexpr int kLanesPerRow = OUT_F32 ? 8 : 4;        // 16 bytes per lane
+    constexpr int kRowsPerStore = kWave / kLanesPerRow;  // 8 or 16
+    constexpr int kUnit = 16 / (int)kOutBytes;           // columns per lane: 4 or 8
+    const int q = lane % kLanesPerRow, rr = lane / kLanesPerRow;
 #pragma unroll
     for (int rs = 0; rs < 2; ++rs) {
-      const unsigned orow = (unsigned)(64 * wave + 32 * rs + c) * (unsigned)V;
 #pragma unroll
       for (int vt = 0; vt < 4; ++vt) {
-        // after the exchange this lane owns columns vs .. vs + 15 of its row
-        const int vs = n0 + 32 * vt + 16 * h;
-        float y[16];
+        // register 4 j + i: column n0 + 32 vt + 8 j + 4 h + i, row c of the tile
+        float tmax = OT_NEG_INF;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const u32x2 r1 = __builtin_amdgcn_permlane32_swap(
-              as_u32(acc[rs][vt][i]), as_u32(acc[rs][vt][8 + i]), false, false);
-          const u32x2 r2 = __builtin_amdgcn_permlane32_swap(
-              as_u32(acc[rs][vt][4 + i]), as_u32(acc[rs][vt][12 + i]), false, false);
-          y[i] = as_f32(r1.x);
-          y[4 + i] = as_f32(r1.y);
-          y[8 + i] = as_f32(r2.x);
-          y[12 + i] = as_f32(r2.y);
-        }
-        unsigned packed[8];
-        if (!OUT_F32) {
+        for (int j = 0; j < 4; ++j) {
+          float y[4];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const unsigned short lo = from_float<E>(y[2 * e]), hi = from_float<E>(y[2 * e + 1]);
-            packed[e] = (unsigned)lo | ((unsigned)hi << 16);
-            y[2 * e] = to_float<E>(lo);
-            y[2 * e + 1] = to_float<E>(hi);
+          for (int i = 0; i < 4; ++i) y[i] = acc[rs][vt][4 * j + i];
+          if (OUT_F32) {
+            const f32x4 t = {y[0], y[1], y[2], y[3]};
+            *reinterpret_cast<f32x4 *>(tile + c * kTilePitch + (8 * j + 4 * h) * 4) = t;
+          } else {
+            const unsigned short b0 = from_float<E>(y[0]), b1 = from_float<E>(y[1]);
+            const unsigned short b2 = from_float<E>(y[2]), b3 = from_float<E>(y[3]);
+            const u32x2 t = {(unsigned)b0 | ((unsigned)b1 << 16), (unsigned)b2 | ((unsigned)b3 << 16)};
+            *reinterpret_cast<u32x2 *>(tile + c * kTilePitch + (8 * j + 4 * h) * 2) = t;
+            y[0] = to_float<E>(b0);
+            y[1] = to_float<E>(b1);
+            y[2] = to_float<E>(b2);
+            y[3] = to_float<E>(b3);
           }
-        }
-        // store: pieces of SV elements; V is a multiple of SV, so a piece is inside the
-        // row or past it as a whole
 #pragma unroll
-        for (int p = 0; p < 16; p += SV) {
-          if (vs + p < V) {
-            const unsigned off = (orow + (unsigned)(vs + p)) * kOutBytes;
-            if (OUT_F32) {
-              if (SV == 4) {
-                const f32x4 t = {y[p], y[p + 1], y[p + 2], y[p + 3]};
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, t), obuf, off, 0, 0);
-              } else if (SV == 2) {
-                const u32x2 t = {as_u32(y[p]), as_u32(y[p + 1])};
-                __builtin_amdgcn_raw_buffer_store_b64(t, obuf, off, 0, 0);
-              } else {
-                __builtin_amdgcn_raw_buffer_store_b32(as_u32(y[p]), obuf, off, 0, 0);
-              }
-            } else {
-              if (SV == 8) {
-                const u32x4 t = {packed[p / 2], packed[p / 2 + 1], packed[p / 2 + 2], packed[p / 2 + 3]};
-                __builtin_amdgcn_raw_buffer_store_b128(t, obuf, off, 0, 0);
-              } else if (SV == 4) {
-                const u32x2 t = {packed[p / 2], packed[p / 2 + 1]};
-                __builtin_amdgcn_raw_buffer_store_b64(t, obuf, off, 0, 0);
-              } else if (SV == 2) {
-                __builtin_amdgcn_raw_buffer_store_b32(packed[p / 2], obuf, off, 0, 0);
-              } else {
-                const unsigned pair = packed[p / 2];
-                __builtin_amdgcn_raw_buffer_store_b16(
-                    (unsigned short)((p & 1) ? (pair >> 16) : (pair & 0xffffu)), obuf, off, 0, 0);
-              }
-            }
+          for (int i = 0; i < 4; ++i) {
+            if (ragged) y[i] = (n0 + 32 * vt + 8 * j + 4 * h + i < V) ? y[i] : OT_NEG_INF;
+            acc[rs][vt][4 * j + i] = y[i];
+            tmax = fmaxf(tmax, y[i]);
           }
         }
         // running (max, sum) of the row over this lane's share of the columns
-        if (ragged) {
-#pragma unroll
-          for (int e = 0; e < 16; ++e) y[e] = (vs + e < V) ? y[e] : OT_NEG_INF;
-        }
-        float tmax = y[0];
-#pragma unroll
-        for (int e = 1; e < 16; ++e) tmax = fmaxf(tmax, y[e]);
         const float nm = fmaxf(m_run[rs], tmax);
         const float ref = __builtin_isinf(nm) ? 0.f : nm;
         const float oldref = __builtin_isinf(m_run[rs]) ? 0.f : m_run[rs];
-        float s = (s_run[rs] == 0.f) ? 0.f : s_run[rs] * exp_fast(oldref - ref);
+        float sum = (s_run[rs] == 0.f) ? 0.f : s_run[rs] * exp_fast(oldref - ref);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s += exp_fast(y[e] - ref);
-        s_run[rs] = s;
+        for (int e = 0; e < 16; ++e) sum += exp_fast(acc[rs][vt][e] - ref);
+        s_run[rs] = sum;
         m_run[rs] = nm;
+        // the tile's rows leave as contiguous pieces
+#pragma unroll
+        for (int it = 0; it < 32 / kRowsPerStore; ++it) {
+          const int trow = it * kRowsPerStore + rr;
+          const u32x4 t = *reinterpret_cast<const u32x4 *>(tile + trow * kTilePitch + q * 16);
+          const int col = n0 + 32 * vt + q * kUnit;
+          const unsigned off =
+              ((unsigned)(64 * wm + 32 * rs + trow) * (unsigned)V + (unsigned)col) * kOutBytes;
+          if (SV == kUnit) {
+            if (col < V) __builtin_amdgcn_raw_buffer_store_b128(t, obuf, off, 0, 0);
+          } else if (SV * kOutBytes == 8) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+              const u32x2 t2 = {t[2 * p], t[2 * p + 1]};
+              if (col + p * SV < V) __builtin_amdgcn_raw_buffer_store_b64(t2, obuf, off + 8u * p, 0, 0);
+            }
+          } else if (SV * kOutBytes == 4) {
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+              if (col + p * SV < V) __builtin_amdgcn_raw_buffer_store_b32(t[p], obuf, off + 4u * p, 0, 0);
+          } else {  // single 2-byte elements
+#pragma unroll
+            for (int p = 0; p < 8; ++p)
+              if (col + p < V)
+                __builtin_amdgcn_raw_buffer_store_b16(
+                    (unsigned short)((p & 1) ? (t[p / 2] >> 16) : (t[p / 2] & 0xffffu)), obuf,
+                    off + 2u * p, 0, 0);
+          }
+        }
       }
     }
   }
 
-  // a row's two lanes (c, c + 32) merge their halves; the lower one writes
+  // a row's shares meet: the two lanes (c, c + 32) of each of its 2 waves
+  auto merge = [](float m1, float s1, float m2, float s2, float &m, float &sum) {
+    m = fmaxf(m1, m2);
+    const float ref = __builtin_isinf(m) ? 0.f : m;
+    const float r1 = __builtin_isinf(m1) ? 0.f : m1, r2 = __builtin_isinf(m2) ? 0.f : m2;
+    sum = ((s1 == 0.f) ? 0.f : s1 * exp_fast(r1 - ref)) + ((s2 == 0.f) ? 0.f : s2 * exp_fast(r2 - ref));
+  };
 #pragma unroll
   for (int rs = 0; rs < 2; ++rs) {
     const float m2 = __shfl_xor(m_run[rs], 32, kWave), s2 = __shfl_xor(s_run[rs], 32, kWave);
-    const float nm = fmaxf(m_run[rs], m2);
-    const float ref = __builtin_isinf(nm) ? 0.f : nm;
-    const float r1 = __builtin_isinf(m_run[rs]) ? 0.f : m_run[rs];
-    const float r2 = __builtin_isinf(m2) ? 0.f : m2;
-    const float s = ((s_run[rs] == 0.f) ? 0.f : s_run[rs] * exp_fast(r1 - ref)) +
-                    ((s2 == 0.f) ? 0.f : s2 * exp_fast(r2 - ref));
-    const unsigned r = (unsigned)(64 * wave + 32 * rs + c);
-    if (h == 0 && r < nrows) den[row0 + r] = logf(s) + ref;
+    float m, sum;
+    merge(m_run[rs], s_run[rs], m2, s2, m, sum);
+    if (h == 0) s_part[wn][64 * wm + 32 * rs + c] = make_float2(m, sum);
+  }
+  __syncthreads();
+  if (tid < kProjRows && (unsigned)tid < nrows) {
+    float m = s_part[0][tid].x, sum = s_part[0][tid].y;
+    merge(m, sum, s_part[1][tid].x, s_part[1][tid].y, m, sum);
+    den[row0 + tid] = logf(sum) + (__builtin_isinf(m) ? 0.f : m);
   }
 }
 
@@ -312,7 +352,7 @@ static int launch_project(const unsigned short *x, const unsigned short *w, cons
   while (sv > 1 && (V % sv != 0 || (reinterpret_cast<uintptr_t>(logits) & (uintptr_t)(sv * esize - 1))))
     sv >>= 1;
 #define OT_LAUNCH_PROJ(SV_)                                                                       \
-  hipLaunchKernelGGL((joiner_project_kernel<E, OUT_F32, SV_>), dim3((unsigned)blocks), dim3(256), \
+  hipLaunchKernelGGL((joiner_project_kernel<E, OUT_F32, SV_>), dim3((unsigned)blocks), dim3(kProjThreads), \
                      0, s, x, w, bias, rows, D, V, logits, den)
   switch (sv) {
     case 8: if constexpr (!OUT_F32) { OT_LAUNCH_PROJ(8); } break;
@@ -337,8 +377,9 @@ int ot_joiner_project(const void *x, const void *weight, const float *bias, int3
       (dtype != OT_DTYPE_F16 && dtype != OT_DTYPE_BF16) ||
       (logits_dtype != OT_DTYPE_F32 && logits_dtype != dtype))
     return OT_E_BAD_ARG;
-  // one stage is 32 k-values; offsets inside a workgroup's rows and inside W are 32-bit
-  if (D % kProjK != 0 || (int64_t)V * D * 2 > (int64_t)UINT32_MAX ||
+  // two stages of 32 k-values per turn of the main loop; offsets inside a workgroup's
+  // rows and inside W are 32-bit
+  if (D % (2 * kProjK) != 0 || ((int64_t)V + 2 * kProjCols) * D * 2 > (int64_t)UINT32_MAX ||
       (int64_t)kProjRows * V * 4 > (int64_t)UINT32_MAX || (int64_t)kProjRows * D * 2 > (int64_t)UINT32_MAX)
     return OT_E_BAD_ARG;
   if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(weight) & 15) ||

@@ -15,7 +15,7 @@ input in that layout with Python lists (README.md:166-177)::
 (``activation="tanh"``) with one kernel, and its gradient with one pass over the
 incoming gradient.
 """
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -78,3 +78,52 @@ def pack_joiner(
         encoder_out, decoder_out, logit_lengths, target_lengths,
         "none" if activation is None else activation,
     )
+
+
+class ProjectJoinerFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, float32_logits):
+        logits, den = _optimized_transducer.joiner_project(
+            x=x, weight=weight, bias=bias, float32_logits=float32_logits)
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        ctx.bias_dtype = bias.dtype if bias is not None else None
+        ctx.mark_non_differentiable(den)
+        return logits, den
+
+    @staticmethod
+    def backward(ctx, grad_logits, _grad_den):
+        # plain dense products: the library's kernels
+        x, weight = ctx.saved_tensors
+        g = grad_logits if grad_logits.dtype == x.dtype else grad_logits.to(x.dtype)
+        grad_x = g @ weight if ctx.needs_input_grad[0] else None
+        grad_w = g.t() @ x if ctx.needs_input_grad[1] else None
+        grad_b = None
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            grad_b = grad_logits.sum(0, dtype=torch.float32).to(ctx.bias_dtype)
+        return grad_x, grad_w, grad_b, None
+
+
+def project_joiner(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                   float32_logits: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The joiner's output projection in front of the loss (``logits = linear(x)`` in
+    the reference's README.md:176-177) for a joiner under mixed precision, with
+    the loss's denominators as a by-product.
+
+    Args:
+      x: (sum_i T_i * (U_i + 1), D) float16 or bfloat16, contiguous, D a multiple
+        of 64: the packed joiner activations, e.g. ``pack_joiner(...).to(torch.bfloat16)``.
+      weight: (V, D), dtype of ``x`` (``nn.Linear.weight`` layout).
+      bias: (V,) or None.
+      float32_logits: True: float32 logits (accumulated in float32, never rounded
+        to 16 bits); False: logits in the dtype of ``x``.
+    Returns:
+      (logits, denominators): ``logits`` (rows, V) = x @ weight.T + bias, computed on
+      the matrix cores with float32 accumulation; ``denominators`` (rows,) float32 =
+      ``logits.logsumexp(1)`` of exactly the stored values, taken from the
+      accumulators.  Pass both to ``transducer_loss(logits, ..., from_log_softmax=False,
+      denominators=denominators)``: the loss then reads the logits once, not twice.
+      Differentiable in ``x``, ``weight`` and ``bias`` (the backward products are
+      torch's own); ``denominators`` carries no gradient.
+    """
+    return ProjectJoinerFunction.apply(x, weight, bias, float32_logits)

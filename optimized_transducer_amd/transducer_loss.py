@@ -27,6 +27,8 @@ of ``forward``), and that a loss which is scaled or weighted before
 ``backward()`` (mixed-precision loss scaling, a weighted sum of losses) costs no
 second pass over the gradient.
 """
+from typing import Optional
+
 import torch
 
 from . import _optimized_transducer
@@ -45,6 +47,7 @@ class TransducerLossFunction(torch.autograd.Function):
         one_sym_per_frame: bool,
         reduction: str = "mean",
         defer_gradient: bool = False,
+        denominators: Optional[torch.Tensor] = None,
     ) -> torch.Tensor:
         """See :func:`transducer_loss` for the arguments.
 
@@ -68,6 +71,7 @@ class TransducerLossFunction(torch.autograd.Function):
                 from_log_softmax=from_log_softmax,
                 one_sym_per_frame=one_sym_per_frame,
                 grad_scale=grad_scale,
+                denominators=denominators,
             )
             if coefficients is not None:
                 # saved through autograd: an in-place change of logits before
@@ -85,6 +89,7 @@ class TransducerLossFunction(torch.autograd.Function):
             from_log_softmax=from_log_softmax,
             one_sym_per_frame=one_sym_per_frame,
             grad_scale=grad_scale,
+            denominators=denominators,
         )
 
         # loss = -1 * scores, then .mean() or .sum() (reference transducer_loss.py:145-147)
@@ -96,7 +101,7 @@ class TransducerLossFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, loss_grad):
         assert loss_grad.numel() == 1, loss_grad.numel()
-        no_grads = (None,) * 8  # targets ... defer_gradient
+        no_grads = (None,) * 9  # targets ... denominators
         if ctx.deferred is not None:
             coefficients, from_log_softmax, grad_scale = ctx.deferred
             assert coefficients is not None, "backward through a deferred transducer loss runs once"
@@ -179,6 +184,7 @@ def transducer_loss(
     reduction: str = "mean",
     *,
     defer_gradient: bool = False,
+    denominators: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Transducer loss of a packed batch.
 
@@ -202,6 +208,10 @@ def transducer_loss(
         leaves ``logits`` alone and ``backward`` computes the gradient (into
         the ``logits`` buffer for logits input), already multiplied by the
         upstream gradient.  ``logits`` must not be modified in between.
+      denominators: not in the reference.  The per-row log-sum-exp of
+        ``logits`` (float32, shape (logits.size(0),)) when the caller already
+        has it, as :func:`project_joiner` returns it: the loss then skips its
+        own pass over the logits for it.  Logits input only.
     Returns:
       A 0-dim tensor with the reduced negative log-likelihood.
     """
@@ -215,4 +225,5 @@ def transducer_loss(
         one_sym_per_frame,
         reduction,
         defer_gradient,
+        denominators,
     )

@@ -46,7 +46,7 @@ def _check(x, w, b, out_dtype):
 
 @pytest.mark.parametrize("out", ["f32", "same"])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("rows,D,V", [(700, 64, 500), (256, 32, 128), (1, 512, 37), (513, 96, 1030),
+@pytest.mark.parametrize("rows,D,V", [(700, 64, 500), (256, 64, 128), (1, 512, 37), (513, 192, 1030),
                                       (300, 128, 6), (64, 256, 130)])
 def test_projection_and_denominators(rows, D, V, dtype, out, device):
     rng = np.random.default_rng(rows * 7 + V)
@@ -89,3 +89,60 @@ def test_log_probs_given_denominators(dtype, device):
     got = cabi.log_probs_given_den(xd, torch.from_numpy(den).to(device), dtg, dU, splits, 0).cpu().numpy()
     m = np.isfinite(want)
     assert (got[m] == want[m]).all() and np.isneginf(got[~m]).all()
+
+
+@pytest.mark.parametrize("f32_logits", [True, False])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_python_pipeline_matches_the_unfused_one(dtype, f32_logits, device):
+    """project_joiner + transducer_loss(denominators=...) against torch's linear followed
+    by transducer_loss on the same (rounded) logits: same loss, same gradients."""
+    import optimized_transducer_amd as ot
+    dt = HALF[dtype]
+    rng = np.random.default_rng(17)
+    T, U, tg, _ = helpers.random_batch(rng, 6, 12, 7, 8)
+    rows, D, V = int((T * (U + 1)).sum()), 64, 90
+    tg = (tg % (V - 1) + 1).astype(np.int32)
+    x0, w0, b0 = _inputs(rng, rows, D, V, dt, device)
+    dT, dU, dtg = (torch.from_numpy(a).to(device) for a in (T, U, tg))
+
+    def run(fused):
+        x, w, b = (t.clone().requires_grad_(True) for t in (x0, w0, b0))
+        if fused:
+            logits, den = ot.project_joiner(x, w, b, float32_logits=f32_logits)
+            loss = ot.transducer_loss(logits, dtg, dT, dU, 0, False, reduction="sum", denominators=den)
+        else:
+            logits = torch.nn.functional.linear(x.float(), w.float(), b)
+            if not f32_logits:
+                logits = logits.to(dt)
+            loss = ot.transducer_loss(logits, dtg, dT, dU, 0, False, reduction="sum")
+        (3.0 * loss).backward()
+        return loss.item(), x.grad.float().cpu().numpy(), w.grad.float().cpu().numpy(), b.grad.cpu().numpy()
+
+    lf, gxf, gwf, gbf = run(True)
+    lu, gxu, gwu, gbu = run(False)
+    # logits differ by float32 summation order (and, in 16 bits, by rare one-unit flips)
+    unit = ULP[dt] if not f32_logits else 1e-6
+    assert abs(lf - lu) <= 4 * unit * rows + 1e-4 * abs(lu), (lf, lu)
+    for a, b_ in ((gxf, gxu), (gwf, gwu), (gbf, gbu)):
+        scale = np.abs(b_).max()
+        assert np.abs(a - b_).max() <= (0.02 if dt == torch.bfloat16 else 0.004) * scale + 1e-6, \
+            (np.abs(a - b_).max(), scale)
+
+
+def test_denominators_argument_is_checked(device):
+    import optimized_transducer_amd as ot
+    rng = np.random.default_rng(2)
+    T, U, tg, x = helpers.random_batch(rng, 3, 5, 3, 11)
+    dT, dU, dtg = (torch.from_numpy(a).to(device) for a in (T, U, tg))
+    logits = torch.from_numpy(x).to(device)
+    den = torch.logsumexp(logits, 1)
+    want = ot.transducer_loss(logits.clone(), dtg, dT, dU, 0, False).item()
+    got = ot.transducer_loss(logits.clone(), dtg, dT, dU, 0, False, denominators=den).item()
+    assert abs(got - want) <= 1e-5 * abs(want) + 1e-5
+    with pytest.raises(RuntimeError, match="denominators"):
+        ot.transducer_loss(logits.clone(), dtg, dT, dU, 0, False, denominators=den[:-1].contiguous())
+    with pytest.raises(RuntimeError, match="denominators"):
+        ot.transducer_loss(torch.log_softmax(logits, 1), dtg, dT, dU, 0, True, denominators=den)
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        ot.project_joiner(torch.zeros(4, 32, dtype=torch.bfloat16, device=device),
+                          torch.zeros(5, 32, dtype=torch.bfloat16, device=device))

@@ -69,7 +69,7 @@ def test_python_entry_points_keep_the_reference_signatures():
     assert list(sig.parameters)[:8] == ref_names
     for extra in list(sig.parameters)[8:]:  # additions: keyword only, off by default
         assert sig.parameters[extra].kind is inspect.Parameter.KEYWORD_ONLY
-        assert sig.parameters[extra].default is False
+        assert sig.parameters[extra].default in (False, None)
     assert sig.parameters["one_sym_per_frame"].default is False
     assert sig.parameters["reduction"].default == "mean"
     assert sig.parameters["from_log_softmax"].default is inspect.Parameter.empty
