@@ -191,6 +191,98 @@ def bench_joiner(args):
     print(json.dumps(out), flush=True)
 
 
+def bench_project(args):
+    """Secondary benchmark: the joiner's output projection fused with the loss's
+    denominators (project_joiner, 16-bit activations and weight, matrix cores),
+    followed by the loss forward + backward on its logits; beside it the same step
+    with torch's own projection and the loss's own denominator pass."""
+    import torch
+    import optimized_transducer_amd as ot
+    from optimized_transducer_amd import _optimized_transducer as ext
+
+    dev = torch.device("cuda", 0)
+    w = make_workload(args.workload)
+    K, W, D = args.steps, args.warmup, args.joiner_dim
+    N, R, V = w.N, w.rows, w.V
+    act = torch.bfloat16 if args.logits_dtype != "f16" else torch.float16
+    f32_logits = args.logits_dtype == "f32"
+    gen = torch.Generator(device="cpu").manual_seed(w.seed)
+    x = torch.tanh(torch.randn((R, D), generator=gen)).to(act).to(dev)
+    wt = (torch.randn((V, D), generator=gen) / D ** 0.5).to(act).to(dev)
+    bias = torch.randn((V,), generator=gen).to(dev)
+    targets = torch.from_numpy(w.targets).to(dev)
+    T = torch.from_numpy(w.logit_lengths).to(dev)
+    U = torch.from_numpy(w.target_lengths).to(dev)
+
+    def fused():
+        logits, den = ext.joiner_project(x=x, weight=wt, bias=bias, float32_logits=f32_logits)
+        logits.requires_grad_(True)
+        loss = ot.transducer_loss(logits, targets, T, U, w.blank, False, w.one_sym_per_frame,
+                                  "sum", denominators=den)
+        loss.backward()
+
+    bias_act = bias.to(act)
+
+    def unfused():
+        if f32_logits:
+            logits = torch.mm(x, wt.t(), out_dtype=torch.float32).add_(bias)
+        else:
+            logits = torch.addmm(bias_act, x, wt.t())
+        logits.requires_grad_(True)
+        loss = ot.transducer_loss(logits, targets, T, U, w.blank, False, w.one_sym_per_frame, "sum")
+        loss.backward()
+
+    def timed(step):
+        for _ in range(W):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(K):
+            step()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    elapsed = timed(fused)
+    elapsed_unfused = timed(unfused)
+    flops = 2.0 * R * D * V
+    out = {
+        "metric": "utterances/sec joiner output projection (fused denominators) + transducer loss "
+                  "fwd+bwd; achieved MFMA TFLOP/s of the projection vs peak",
+        "value": N * K / elapsed, "unit": "utterances/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": 1e3 * elapsed / K, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": args.logits_dtype if not f32_logits else "bf16->f32",
+        "data": "synthetic",
+        "config": {"workload": "joiner_projection_of_" + w.name, "N": N, "D": D, "V": V,
+                   "packed_rows": R, "activations": str(act).split(".")[-1],
+                   "logits": "f32" if f32_logits else str(act).split(".")[-1]},
+        "unfused": {"ms_per_step": 1e3 * elapsed_unfused / K,
+                    "what": "torch (hipBLASLt) projection of the same operands, then the loss with "
+                            "its own denominator pass"},
+    }
+    ext.set_profiling(True)
+    for _ in range(K):
+        fused()
+    torch.cuda.synchronize()
+    ext.set_profiling(False)
+    per = {}
+    for name, ms in ext.take_profile():
+        per.setdefault(name, []).append(ms)
+    kernels = {name: {"ms_per_step": sum(ms) / K, "launches_per_step": len(ms) / K}
+               for name, ms in per.items()}
+    t = kernels["joiner_project"]["ms_per_step"]
+    kernels["joiner_project"]["flops"] = flops
+    kernels["joiner_project"]["achieved_TFLOPs"] = flops / (t * 1e-3) / 1e12
+    # bytes the projection cannot avoid: read x and W once, write the logits once
+    min_bytes = 2.0 * R * D + 2.0 * V * D + (4.0 if f32_logits else 2.0) * R * V
+    out["roofline"] = {"bound": "mfma", "kernel": "joiner_project_kernel", "peak": 2500.0,
+                       "achieved": kernels["joiner_project"]["achieved_TFLOPs"], "unit": "TFLOP/s",
+                       "frac": kernels["joiner_project"]["achieved_TFLOPs"] / 2500.0, "traffic": None,
+                       "kernel_ms_per_step": t, "flops_per_step": flops,
+                       "hbm_bound_ms": min_bytes / (HBM_PEAK_GBPS * 1e9) * 1e3}
+    out["kernels"] = kernels
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -205,9 +297,11 @@ def main():
     ap.add_argument("--logits-dtype", default="f32", choices=["f32", "f16", "bf16"],
                     help="element type of the logits; the headline figure uses f32 (the only type "
                          "the reference accepts), f16/bf16 measure the half-precision addition")
-    ap.add_argument("--op", default="loss", choices=["loss", "joiner"],
+    ap.add_argument("--op", default="loss", choices=["loss", "joiner", "project"],
                     help="loss: the headline benchmark; joiner: the packed joiner input "
-                         "(pack_joiner) forward + backward for the workload's lengths")
+                         "(pack_joiner) forward + backward for the workload's lengths; project: "
+                         "the joiner's output projection fused with the denominators "
+                         "(project_joiner), then the loss forward + backward")
     ap.add_argument("--joiner-dim", type=int, default=512)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
@@ -228,6 +322,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     if args.op == "joiner":
         return bench_joiner(args)
+    if args.op == "project":
+        return bench_project(args)
     dev = torch.device("cuda", 0)
     w = make_workload(args.workload)
     K, W = args.steps, args.warmup

@@ -284,5 +284,74 @@ template <> __device__ __forceinline__ unsigned short from_float<BF16>(float x) 
   return __builtin_bit_cast(unsigned short, (__bf16)x);  // round to nearest even
 }
 
+// element i of an array of float (T = float) or of a 2-byte type (T = F16 / BF16)
+template <class T> __device__ __forceinline__ float load_element(const void *p, int64_t i) {
+  return to_float<T>(static_cast<const unsigned short *>(p)[i]);
+}
+template <> __device__ __forceinline__ float load_element<float>(const void *p, int64_t i) {
+  return static_cast<const float *>(p)[i];
+}
+
+// Gather step alone (ComputeLogProbsForLogSoftmax, kernels.cu:62-88; with `den`,
+// ComputeLogProbs, kernels.cu:30-60, for denominators that are already known):
+// lp[row] = (logits[row, blank], logits[row, target(row)]) - (den ? den[row] : 0).
+// Latency-bound (two dependent small reads per row): a thread works on kGatherRows
+// rows at once, starts the reads that need no decoding first and finds its
+// utterances with its own binary searches (row_splits stays in L1), so that nothing
+// in the workgroup waits for anything else.
+constexpr int kGatherRows = 2;
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void gather_rows_kernel(
+    const void *__restrict__ logits, const float *__restrict__ den,
+    const int32_t *__restrict__ targets, const int32_t *__restrict__ target_lengths,
+    const int32_t *__restrict__ row_splits, int N, int targets_cols, int64_t row_begin,
+    int64_t rows, int V, int blank, float *__restrict__ lp) {
+  const int64_t lattice_rows = min(rows, (int64_t)row_splits[N]);
+  int64_t row[kGatherRows];
+  float bl[kGatherRows], d[kGatherRows];
+  int lo[kGatherRows], hi[kGatherRows];
+#pragma unroll
+  for (int k = 0; k < kGatherRows; ++k) {
+    row[k] = row_begin + ((int64_t)blockIdx.x * kGatherRows + k) * kBlock + threadIdx.x;
+    const bool in = row[k] < lattice_rows;
+    bl[k] = in ? load_element<T>(logits, row[k] * (int64_t)V + blank) : 0.f;
+    d[k] = (in && den) ? den[row[k]] : 0.f;
+    lo[k] = 0;
+    hi[k] = N;
+  }
+  // largest b with row_splits[b] <= row, all searches in step
+  for (int width = N; width > 1; width = (width + 1) >> 1) {
+#pragma unroll
+    for (int k = 0; k < kGatherRows; ++k) {
+      if (hi[k] - lo[k] > 1) {
+        const int mid = (lo[k] + hi[k]) >> 1;
+        if ((int64_t)row_splits[mid] <= row[k]) lo[k] = mid; else hi[k] = mid;
+      }
+    }
+  }
+  int col[kGatherRows];
+#pragma unroll
+  for (int k = 0; k < kGatherRows; ++k) {
+    col[k] = -1;
+    if (row[k] < lattice_rows) {
+      const int b = lo[k];
+      const int U = target_lengths[b];
+      const int u1 = U + 1 > 0 ? U + 1 : 1;
+      const int u = (int)(row[k] - row_splits[b]) % u1;
+      if (u < U && u < targets_cols) col[k] = targets[(int64_t)b * targets_cols + u];
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kGatherRows; ++k) {
+    if (row[k] < lattice_rows) {
+      float sym = OT_NEG_INF;
+      if ((unsigned)col[k] < (unsigned)V)
+        sym = load_element<T>(logits, row[k] * (int64_t)V + col[k]) - d[k];
+      reinterpret_cast<float2 *>(lp)[row[k]] = make_float2(bl[k] - d[k], sym);
+    }
+  }
+}
+
 }  // namespace ot
 #endif  // OT_DEVICE_HIP_H_

@@ -5,7 +5,7 @@
 //   prepare_kernel        row offsets + batch facts      cuda.cu:411-414, transducer-loss.cc:49-62
 //   row_ids_kernel        row -> utterance               cuda.cu:40-59 (moderngpu load_balance_search)
 //   lse_gather_kernel     per-row logsumexp + gather     cuda.cu:427 + kernels.cu:30-60
-//   gather_kernel         gather only (log-softmax in)   kernels.cu:62-88
+//   gather_rows_kernel    gather only (log-softmax in)   kernels.cu:62-88  (ot_device.hip.h)
 //   alpha_beta_kernel     lattice DP, both directions    kernels.cu:200-313, 415-519
 //   row_coeff_kernel      per-row part of the gradients  kernels.cu:522-779
 //   grad_flat_kernel      (rows, V) pass of the gradients kernels.cu:522-779
@@ -292,61 +292,6 @@ __global__ __launch_bounds__(kBlock) void lse_gather_kernel(
   const int nlp = 2 * (int)max((int64_t)0, min((int64_t)nrows, lattice_rows - row_first));
   for (int i = threadIdx.x; i < nrows; i += kBlock) den[row_first + i] = s_den[i];
   for (int i = threadIdx.x; i < nlp; i += kBlock) lp[2 * row_first + i] = s_lp[i];
-}
-
-// log-softmax input: no denominator, lp is the two gathered values themselves.
-// Latency-bound (two dependent 4-byte reads per 4V-byte row): a thread works on
-// kGatherRows rows at once, starts the reads that need no decoding first and finds
-// its utterances with its own binary searches (row_splits stays in L1), so that
-// nothing in the workgroup waits for anything else.
-constexpr int kGatherRows = 2;
-
-__global__ __launch_bounds__(kBlock) void gather_kernel(
-    const float *__restrict__ logits, const int32_t *__restrict__ targets,
-    const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
-    int N, int targets_cols, int64_t row_begin, int64_t rows, int V, int blank,
-    float *__restrict__ lp) {
-  const int64_t lattice_rows = min(rows, (int64_t)row_splits[N]);
-  int64_t row[kGatherRows];
-  float bl[kGatherRows];
-  int lo[kGatherRows], hi[kGatherRows];
-#pragma unroll
-  for (int k = 0; k < kGatherRows; ++k) {
-    row[k] = row_begin + ((int64_t)blockIdx.x * kGatherRows + k) * kBlock + threadIdx.x;
-    bl[k] = row[k] < lattice_rows ? logits[row[k] * (int64_t)V + blank] : 0.f;
-    lo[k] = 0;
-    hi[k] = N;
-  }
-  // largest b with row_splits[b] <= row, all searches in step
-  for (int width = N; width > 1; width = (width + 1) >> 1) {
-#pragma unroll
-    for (int k = 0; k < kGatherRows; ++k) {
-      if (hi[k] - lo[k] > 1) {
-        const int mid = (lo[k] + hi[k]) >> 1;
-        if ((int64_t)row_splits[mid] <= row[k]) lo[k] = mid; else hi[k] = mid;
-      }
-    }
-  }
-  int col[kGatherRows];
-#pragma unroll
-  for (int k = 0; k < kGatherRows; ++k) {
-    col[k] = -1;
-    if (row[k] < lattice_rows) {
-      const int b = lo[k];
-      const int U = target_lengths[b];
-      const int u1 = U + 1 > 0 ? U + 1 : 1;
-      const int u = (int)(row[k] - row_splits[b]) % u1;
-      if (u < U && u < targets_cols) col[k] = targets[(int64_t)b * targets_cols + u];
-    }
-  }
-#pragma unroll
-  for (int k = 0; k < kGatherRows; ++k) {
-    if (row[k] < lattice_rows) {
-      float sym = OT_NEG_INF;
-      if ((unsigned)col[k] < (unsigned)V) sym = logits[row[k] * (int64_t)V + col[k]];
-      reinterpret_cast<float2 *>(lp)[row[k]] = make_float2(bl[k], sym);
-    }
-  }
 }
 
 // ---------------------------------------------------------------------------
@@ -970,9 +915,10 @@ int ot_log_probs_range(const float *logits, const int32_t *targets, const int32_
   if (from_log_softmax) {
     const int64_t per_block = (int64_t)kGatherRows * kBlock;
     const unsigned blocks = (unsigned)((count + per_block - 1) / per_block);
-    hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(kBlock), 0, s, logits, targets,
-                       target_lengths, row_splits, N, targets_cols, row_begin, row_end, V, blank,
-                       lp);
+    hipLaunchKernelGGL(gather_rows_kernel<float>, dim3(blocks), dim3(kBlock), 0, s,
+                       static_cast<const void *>(logits), static_cast<const float *>(nullptr),
+                       targets, target_lengths, row_splits, N, targets_cols, row_begin, row_end, V,
+                       blank, lp);
     return launch_status();
   }
   const RowTiling t = pick_tiling(V, is_aligned16(logits));

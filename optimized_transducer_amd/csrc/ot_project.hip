@@ -310,35 +310,6 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
   }
 }
 
-// lp = (logits[row, blank], logits[row, target]) - den[row] for denominators that
-// are already known (cpu.cc:52-100 without its log-sum-exp); T = float or a 2-byte type
-template <class E, bool IS_F32>
-__global__ __launch_bounds__(kBlock) void gather_given_den_kernel(
-    const void *__restrict__ logits, const float *__restrict__ den,
-    const int32_t *__restrict__ targets, const int32_t *__restrict__ target_lengths,
-    const int32_t *__restrict__ row_splits, int N, int targets_cols, int V, int blank,
-    float *__restrict__ lp) {
-  const int64_t lattice_rows = row_splits[N];
-  const int64_t row = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (row >= lattice_rows) return;
-  auto value = [&](int col) -> float {
-    const int64_t i = row * (int64_t)V + col;
-    if (IS_F32) return static_cast<const float *>(logits)[i];
-    return to_float<E>(static_cast<const unsigned short *>(logits)[i]);
-  };
-  const float d = den[row];
-  const float bl = value(blank) - d;
-  const int b = find_utterance(row_splits, N, row);
-  const int U = target_lengths[b];
-  const int u = (int)(row - row_splits[b]) % (U + 1 > 0 ? U + 1 : 1);
-  float sym = OT_NEG_INF;
-  if (u < U && u < targets_cols) {
-    const int col = targets[(int64_t)b * targets_cols + u];
-    if ((unsigned)col < (unsigned)V) sym = value(col) - d;
-  }
-  reinterpret_cast<float2 *>(lp)[row] = make_float2(bl, sym);
-}
-
 static inline int launch_status() { return (int)hipGetLastError(); }
 
 template <class E, bool OUT_F32>
@@ -409,13 +380,14 @@ int ot_log_probs_given_den(const void *logits, int32_t dtype, const float *den,
     return OT_E_BAD_ARG;
   if (reinterpret_cast<uintptr_t>(logits) & (dtype == OT_DTYPE_F32 ? 3 : 1)) return OT_E_MISALIGNED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid((unsigned)((rows + kBlock - 1) / kBlock));
-#define OT_LAUNCH_GGD(E_, F32_)                                                                   \
-  hipLaunchKernelGGL((gather_given_den_kernel<E_, F32_>), grid, dim3(kBlock), 0, s, logits, den,  \
-                     targets, target_lengths, row_splits, N, targets_cols, V, blank, lp)
-  if (dtype == OT_DTYPE_F32) OT_LAUNCH_GGD(BF16, true);
-  else if (dtype == OT_DTYPE_F16) OT_LAUNCH_GGD(F16, false);
-  else OT_LAUNCH_GGD(BF16, false);
+  const int64_t per_block = (int64_t)kGatherRows * kBlock;
+  const dim3 grid((unsigned)((rows + per_block - 1) / per_block));
+#define OT_LAUNCH_GGD(T_)                                                                        \
+  hipLaunchKernelGGL(gather_rows_kernel<T_>, grid, dim3(kBlock), 0, s, logits, den, targets,      \
+                     target_lengths, row_splits, N, targets_cols, (int64_t)0, rows, V, blank, lp)
+  if (dtype == OT_DTYPE_F32) OT_LAUNCH_GGD(float);
+  else if (dtype == OT_DTYPE_F16) OT_LAUNCH_GGD(F16);
+  else OT_LAUNCH_GGD(BF16);
 #undef OT_LAUNCH_GGD
   return launch_status();
 }
