@@ -45,6 +45,9 @@ constexpr int kProjRows = 128;     // packed rows per workgroup (2 waves)
 constexpr int kProjCols = 256;     // vocabulary columns per pass (2 waves)
 constexpr int kProjK = 32;         // k-values per LDS stage
 constexpr int kProjThreads = 256;
+// ordinary (cached) stores: rows whose pitch is not a multiple of 128 bytes are written in
+// partial lines, for which the non-temporal policies are 20-90 % slower here
+constexpr int kProjStoreAux = 0;
 constexpr int kProjWBytes = kProjCols * kProjK * 2;
 constexpr int kProjXBytes = kProjRows * kProjK * 2;
 constexpr int kProjStageBytes = kProjWBytes + kProjXBytes;
@@ -185,10 +188,14 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
         const f32x4 b4 = __builtin_bit_cast(
             f32x4, __builtin_amdgcn_raw_buffer_load_b128(
                        bbuf, (unsigned)(n0 + 32 * vt + 8 * j + 4 * h) * 4u, 0, 0));
+        // vocabulary entries past V start from -inf and stay there (their rows of W read
+        // as zeros), so they drop out of the log-sum-exp without a mask in the epilogue
+        const int v0 = n0 + 32 * vt + 8 * j + 4 * h;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          acc[0][vt][4 * j + i] = b4[i];
-          acc[1][vt][4 * j + i] = b4[i];
+          const float start = (v0 + i < V) ? b4[i] : OT_NEG_INF;
+          acc[0][vt][4 * j + i] = start;
+          acc[1][vt][4 * j + i] = start;
         }
       }
     for (int kk = 0; kk < ksteps; kk += 2) {
@@ -208,7 +215,6 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
     // A tile's values go through a wave-private LDS tile (32 rows x 32 columns) that
     // turns the accumulator layout (one 16-byte piece per lane and row) into whole
     // 128-byte (64-byte for 2-byte logits) pieces of rows per store instruction.
-    const bool ragged = n0 + 128 > V;  // this wave's columns may reach past V
     unsigned char *tile = s_tile + wave * kProjTileBytes;
     constexpr int kTilePitch = OUT_F32 ? kProjTilePitch : kProjTilePitch / 2 + 8;  // 144 / 80 bytes
     constexpr int kLanesPerRow = OUT_F32 ? 8 : 4;        // 16 bytes per lane
@@ -241,7 +247,6 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
           }
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            if (ragged) y[i] = (n0 + 32 * vt + 8 * j + 4 * h + i < V) ? y[i] : OT_NEG_INF;
             acc[rs][vt][4 * j + i] = y[i];
             tmax = fmaxf(tmax, y[i]);
           }
@@ -251,8 +256,12 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
         const float ref = __builtin_isinf(nm) ? 0.f : nm;
         const float oldref = __builtin_isinf(m_run[rs]) ? 0.f : m_run[rs];
         float sum = (s_run[rs] == 0.f) ? 0.f : s_run[rs] * exp_fast(oldref - ref);
+        // exp(y - ref) = 2^(y * log2(e) - ref * log2(e)): one fused multiply-add per term
+        constexpr float kLog2e = 1.44269502162933349609375f;
+        const float shift = -ref * kLog2e;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) sum += exp_fast(acc[rs][vt][e] - ref);
+        for (int e = 0; e < 16; ++e)
+          sum += __builtin_amdgcn_exp2f(__builtin_fmaf(acc[rs][vt][e], kLog2e, shift));
         s_run[rs] = sum;
         m_run[rs] = nm;
         // the tile's rows leave as contiguous pieces
@@ -264,12 +273,12 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
           const unsigned off =
               ((unsigned)(64 * wm + 32 * rs + trow) * (unsigned)V + (unsigned)col) * kOutBytes;
           if (SV == kUnit) {
-            if (col < V) __builtin_amdgcn_raw_buffer_store_b128(t, obuf, off, 0, 0);
+            if (col < V) __builtin_amdgcn_raw_buffer_store_b128(t, obuf, off, 0, kProjStoreAux);
           } else if (SV * kOutBytes == 8) {
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
               const u32x2 t2 = {t[2 * p], t[2 * p + 1]};
-              if (col + p * SV < V) __builtin_amdgcn_raw_buffer_store_b64(t2, obuf, off + 8u * p, 0, 0);
+              if (col + p * SV < V) __builtin_amdgcn_raw_buffer_store_b64(t2, obuf, off + 8u * p, 0, kProjStoreAux);
             }
           } else if (SV * kOutBytes == 4) {
 #pragma unroll
