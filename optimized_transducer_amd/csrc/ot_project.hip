@@ -86,6 +86,7 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
     float *__restrict__ den) {
   __shared__ __attribute__((aligned(16))) unsigned char s_stage[2 * kProjStageBytes];
   __shared__ float2 s_part[2][kProjRows];
+  __shared__ __attribute__((aligned(16))) float s_bias[kProjCols];  // the pass's starting values
   __shared__ __attribute__((aligned(16))) unsigned char s_tile[4 * kProjTileBytes];
   constexpr unsigned kOutBytes = OUT_F32 ? 4u : 2u;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -173,6 +174,13 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
 
   float m_run[2] = {OT_NEG_INF, OT_NEG_INF}, s_run[2] = {0.f, 0.f};
   ProjStage set_a, set_b;
+  // vocabulary entries past V start from -inf and stay there (their rows of W read as
+  // zeros), so they drop out of the log-sum-exp without a mask in the epilogue
+  auto starting_value = [&](int v) -> float {
+    const float b = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, (unsigned)v * 4u, 0, 0));
+    return v < V ? b : OT_NEG_INF;
+  };
+  s_bias[tid] = starting_value(tid);
   load_stage(set_a);
   load_stage(set_b);
   store_stage(set_a, 0);
@@ -180,22 +188,19 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
   for (int pass = 0; pass < npasses; ++pass) {
     const int n0 = pass * kProjCols + 128 * wn;  // first column of this wave in the pass
     // accumulators start from the bias: tile (rs, vt), register 4 j + i holds vocabulary
-    // entry n0 + 32 vt + 8 j + 4 h + i of packed row 64 wm + 32 rs + c
+    // entry n0 + 32 vt + 8 j + 4 h + i of packed row 64 wm + 32 rs + c.  The pass's
+    // starting values come through LDS (written before the previous pass's stores
+    // were issued): a global load here would have to wait for those stores as well.
+    lds_barrier();
 #pragma unroll
     for (int vt = 0; vt < 4; ++vt)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const f32x4 b4 = __builtin_bit_cast(
-            f32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                       bbuf, (unsigned)(n0 + 32 * vt + 8 * j + 4 * h) * 4u, 0, 0));
-        // vocabulary entries past V start from -inf and stay there (their rows of W read
-        // as zeros), so they drop out of the log-sum-exp without a mask in the epilogue
-        const int v0 = n0 + 32 * vt + 8 * j + 4 * h;
+        const f32x4 b4 = *reinterpret_cast<const f32x4 *>(&s_bias[128 * wn + 32 * vt + 8 * j + 4 * h]);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float start = (v0 + i < V) ? b4[i] : OT_NEG_INF;
-          acc[0][vt][4 * j + i] = start;
-          acc[1][vt][4 * j + i] = start;
+          acc[0][vt][4 * j + i] = b4[i];
+          acc[1][vt][4 * j + i] = b4[i];
         }
       }
     for (int kk = 0; kk < ksteps; kk += 2) {
@@ -216,6 +221,7 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
     // turns the accumulator layout (one 16-byte piece per lane and row) into whole
     // 128-byte (64-byte for 2-byte logits) pieces of rows per store instruction.
     unsigned char *tile = s_tile + wave * kProjTileBytes;
+    if (pass + 1 < npasses) s_bias[tid] = starting_value((pass + 1) * kProjCols + tid);
     constexpr int kTilePitch = OUT_F32 ? kProjTilePitch : kProjTilePitch / 2 + 8;  // 144 / 80 bytes
     constexpr int kLanesPerRow = OUT_F32 ? 8 : 4;        // 16 bytes per lane
     constexpr int kRowsPerStore = kWave / kLanesPerRow;  // 8 or 16
