@@ -92,15 +92,20 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int c = lane & 31, h = lane >> 5;
-  const int64_t row0 = (int64_t)blockIdx.x * kProjRows;
-  const unsigned nrows = (unsigned)min((int64_t)kProjRows, rows - row0);
-  // the workgroup's rows, the weight and the bias as raw buffers: rows past the
-  // array and vocabulary entries past V read as zeros, stores to them vanish
-  const __amdgpu_buffer_rsrc_t xbuf = make_buffer(x + row0 * D, nrows * (unsigned)D * 2u);
+  // Persistent workgroups: workgroup g takes the 128-row tiles g, g + gridDim.x, ...;
+  // the loads of the next tile's first stages are already in flight while the current
+  // tile's last pass is stored.
+  const int64_t ntiles = (rows + kProjRows - 1) / kProjRows;
+  // the weight and the bias as raw buffers: vocabulary entries past V read as zeros
   const __amdgpu_buffer_rsrc_t wbuf = make_buffer(w, (unsigned)V * (unsigned)D * 2u);
   const __amdgpu_buffer_rsrc_t bbuf = make_buffer(bias ? bias : den, bias ? (unsigned)V * 4u : 0u);
-  const __amdgpu_buffer_rsrc_t obuf =
-      make_buffer(static_cast<char *>(logits) + row0 * V * kOutBytes, nrows * (unsigned)V * kOutBytes);
+  // a tile's rows of x as a raw buffer: rows past the array (and whole tiles past the
+  // last one) read as zeros
+  auto x_tile = [&](int64_t tile) {
+    const int64_t r0 = min(tile, ntiles) * kProjRows;
+    const unsigned n = (unsigned)max((int64_t)0, min((int64_t)kProjRows, rows - r0));
+    return make_buffer(x + min(r0, rows - 1) * D, n * (unsigned)D * 2u);
+  };
 
   // stage copy: a stage is 32 k-values = 4 chunks of 16 bytes per row; chunk cc of
   // row r lives in slot 4 r + (cc ^ ((r >> 2) & 3)).  Thread t moves pieces
@@ -127,7 +132,9 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
   // Loads past the last stage are issued all the same (W reads as zeros there, x is
   // re-read): with a branch around them the number of loads in flight would not be
   // known at compile time and every wait would have to drain them all.
+  int64_t load_tile = blockIdx.x;
   int load_pass = 0, load_kk = 0;
+  __amdgpu_buffer_rsrc_t xbuf = x_tile(load_tile);
   auto load_stage = [&](ProjStage &st) {
     const unsigned wbase =
         ((unsigned)(load_pass * kProjCols) * (unsigned)D + (unsigned)(load_kk * kProjK)) * 2u;
@@ -140,7 +147,11 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
           xbuf, piece_src, (unsigned)(load_kk * kProjK) * 2u + q * piece_src_step, 0);
     if (++load_kk == ksteps) {
       load_kk = 0;
-      ++load_pass;
+      if (++load_pass == npasses) {
+        load_pass = 0;
+        load_tile += gridDim.x;
+        xbuf = x_tile(load_tile);
+      }
     }
   };
   auto store_stage = [&](const ProjStage &st, int buf) {
@@ -172,7 +183,6 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
     }
   };
 
-  float m_run[2] = {OT_NEG_INF, OT_NEG_INF}, s_run[2] = {0.f, 0.f};
   ProjStage set_a, set_b;
   // vocabulary entries past V start from -inf and stay there (their rows of W read as
   // zeros), so they drop out of the log-sum-exp without a mask in the epilogue
@@ -185,6 +195,13 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
   load_stage(set_b);
   store_stage(set_a, 0);
   load_stage(set_a);
+  for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+  const int64_t row0 = tile * kProjRows;
+  const unsigned nrows = (unsigned)min((int64_t)kProjRows, rows - row0);
+  // stores to rows past the array vanish
+  const __amdgpu_buffer_rsrc_t obuf =
+      make_buffer(static_cast<char *>(logits) + row0 * V * kOutBytes, nrows * (unsigned)V * kOutBytes);
+  float m_run[2] = {OT_NEG_INF, OT_NEG_INF}, s_run[2] = {0.f, 0.f};
   for (int pass = 0; pass < npasses; ++pass) {
     const int n0 = pass * kProjCols + 128 * wn;  // first column of this wave in the pass
     // accumulators start from the bias: tile (rs, vt), register 4 j + i holds vocabulary
@@ -221,7 +238,9 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
     // turns the accumulator layout (one 16-byte piece per lane and row) into whole
     // 128-byte (64-byte for 2-byte logits) pieces of rows per store instruction.
     unsigned char *tile = s_tile + wave * kProjTileBytes;
-    if (pass + 1 < npasses) s_bias[tid] = starting_value((pass + 1) * kProjCols + tid);
+    // starting values of the next pass (of the next tile after the last one), fetched
+    // before this pass's stores are issued
+    if (npasses > 1) s_bias[tid] = starting_value((pass + 1 < npasses ? pass + 1 : 0) * kProjCols + tid);
     constexpr int kTilePitch = OUT_F32 ? kProjTilePitch : kProjTilePitch / 2 + 8;  // 144 / 80 bytes
     constexpr int kLanesPerRow = OUT_F32 ? 8 : 4;        // 16 bytes per lane
     constexpr int kRowsPerStore = kWave / kLanesPerRow;  // 8 or 16
@@ -317,12 +336,13 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
     merge(m_run[rs], s_run[rs], m2, s2, m, sum);
     if (h == 0) s_part[wn][64 * wm + 32 * rs + c] = make_float2(m, sum);
   }
-  __syncthreads();
+  lds_barrier();  // LDS only: the tile's stores stay in flight
   if (tid < kProjRows && (unsigned)tid < nrows) {
     float m = s_part[0][tid].x, sum = s_part[0][tid].y;
     merge(m, sum, s_part[1][tid].x, s_part[1][tid].y, m, sum);
     den[row0 + tid] = logf(sum) + (__builtin_isinf(m) ? 0.f : m);
   }
+  }  // tiles
 }
 
 static inline int launch_status() { return (int)hipGetLastError(); }
@@ -331,8 +351,13 @@ template <class E, bool OUT_F32>
 static int launch_project(const unsigned short *x, const unsigned short *w, const float *bias,
                           int64_t rows, int32_t D, int32_t V, void *logits, float *den,
                           hipStream_t s) {
-  const int64_t blocks = (rows + kProjRows - 1) / kProjRows;
-  if (blocks > INT32_MAX) return OT_E_BAD_ARG;
+  // two resident workgroups per compute unit walk over the 128-row tiles
+  int device = 0, cus = 0;
+  if (hipGetDevice(&device) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
+    return OT_E_BAD_ARG;
+  const int64_t tiles = (rows + kProjRows - 1) / kProjRows;
+  const int64_t blocks = tiles < 2 * (int64_t)cus ? tiles : 2 * (int64_t)cus;
   const unsigned esize = OUT_F32 ? 4u : 2u;
   int sv = (int)(16u / esize);  // elements per store
   while (sv > 1 && (V % sv != 0 || (reinterpret_cast<uintptr_t>(logits) & (uintptr_t)(sv * esize - 1))))
