@@ -400,3 +400,24 @@ def test_pack_joiner_oracle_matches_the_readme_recipe_and_its_autograd(activatio
     # float32 evaluation of the forward agrees with float64 to rounding
     got32 = oracle.pack_joiner(enc.astype(np.float32), dec.astype(np.float32), T, U, activation)
     assert got32.dtype == np.float32 and np.allclose(got32, got, rtol=1e-6, atol=1e-6)
+
+
+def test_project_joiner_oracle_is_the_linear_layer_of_the_readme():
+    """README.md:176-177 projects the packed activations with nn.Linear: pinned against
+    torch's float64 linear, against explicit sums on a tiny case, and by two properties a
+    transposed weight or a dropped bias would break (identity weight, zero input)."""
+    rng = np.random.default_rng(23)
+    x = rng.standard_normal((9, 6))
+    w = rng.standard_normal((4, 6))
+    b = rng.standard_normal(4)
+    got, mag = oracle.project_joiner(x, w, b)
+    want = torch.nn.functional.linear(torch.tensor(x), torch.tensor(w), torch.tensor(b)).numpy()
+    assert got.shape == (9, 4) and np.allclose(got, want, rtol=1e-14, atol=1e-14)
+    for r, v in ((0, 0), (5, 3), (8, 1)):
+        terms = [x[r, k] * w[v, k] for k in range(6)]
+        assert abs(got[r, v] - (sum(terms) + b[v])) < 1e-13
+        assert abs(mag[r, v] - (sum(abs(t) for t in terms) + abs(b[v]))) < 1e-13
+    eye, _ = oracle.project_joiner(x, np.eye(6))
+    assert np.array_equal(eye, x)
+    zero, zmag = oracle.project_joiner(np.zeros((3, 6)), w, b)
+    assert np.array_equal(zero, np.tile(b, (3, 1))) and np.array_equal(zmag, np.tile(np.abs(b), (3, 1)))
