@@ -315,7 +315,7 @@ int ot_scale_by_device_scalar_half(void *x, int32_t dtype, int64_t n,
  * the denominators (ot_log_probs_given_den instead of ot_log_probs).
  *
  * x (rows, D) and weight (V, D) row-major of `dtype` (OT_DTYPE_F16 or
- * OT_DTYPE_BF16), 16-byte aligned, D a multiple of 32; bias (V) float32 or
+ * OT_DTYPE_BF16), 16-byte aligned, D a multiple of 64; bias (V) float32 or
  * NULL; logits (rows, V) of logits_dtype = OT_DTYPE_F32 or `dtype`;
  * den (rows) float32. */
 int ot_joiner_project(const void *x, const void *weight, const float *bias,
