@@ -124,11 +124,13 @@ def bench_joiner(args):
     dec = dec_h.to(dev).requires_grad_(True)
     T = torch.from_numpy(w.logit_lengths).to(dev)
     U = torch.from_numpy(w.target_lengths).to(dev)
-    g = torch.randn((R, D), device=dev)
+    out_dtype = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[args.logits_dtype]
+    esize = 4 if out_dtype == torch.float32 else 2
+    g = torch.randn((R, D), device=dev).to(out_dtype)
 
     def step():
         enc.grad = dec.grad = None
-        x = ot.pack_joiner(enc, dec, T, U, activation="tanh")
+        x = ot.pack_joiner(enc, dec, T, U, activation="tanh", out_dtype=out_dtype)
         x.backward(g)
 
     for _ in range(W):
@@ -143,9 +145,10 @@ def bench_joiner(args):
         "metric": "utterances/sec packed joiner input (tanh) fwd+bwd; achieved HBM GB/s vs peak",
         "value": N * K / elapsed, "unit": "utterances/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": 1e3 * elapsed / K, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32" if esize == 4 else "f32->" + args.logits_dtype,
+        "data": "synthetic",
         "config": {"workload": "joiner_input_of_" + w.name, "N": N, "D": D, "packed_rows": R,
-                   "T_max": Tm, "U1_max": U1m, "activation": "tanh", "packed_bytes": 4 * R * D},
+                   "T_max": Tm, "U1_max": U1m, "activation": "tanh", "packed_bytes": esize * R * D},
     }
     ext.set_profiling(True)
     for _ in range(K):
@@ -157,7 +160,7 @@ def bench_joiner(args):
         per.setdefault(name, []).append(ms)
     # pack: writes (rows, D) once; unpack: reads (rows, D) once and
     # writes + re-reads one partial decoder sum per 16 frames
-    alg = {"joiner_pack": 4 * D * R, "joiner_unpack_grad": 4 * D * R + 2 * (4 * D * R // 16)}
+    alg = {"joiner_pack": esize * D * R, "joiner_unpack_grad": 4 * D * R + 2 * (4 * D * R // 16)}
     kernels = {}
     for name, ms in per.items():
         per_step = sum(ms) / K

@@ -303,6 +303,18 @@ int ot_gradient_apply_half(const void *logits, int32_t dtype,
 int ot_scale_by_device_scalar_half(void *x, int32_t dtype, int64_t n,
                                    const float *factor, void *stream);
 
+/* ot_joiner_pack with the output rounded (to nearest even) to out_dtype =
+ * OT_DTYPE_F16 or OT_DTYPE_BF16: the activations of a joiner whose projection
+ * runs in 16 bits (ot_joiner_project), without a float32 array and a cast pass
+ * in between.  enc and dec stay float32; D a multiple of 8, enc / dec / out
+ * 16-byte aligned. */
+int ot_joiner_pack_half(const float *enc, const float *dec,
+                        const int32_t *logit_lengths,
+                        const int32_t *target_lengths,
+                        const int32_t *row_splits, int32_t N, int32_t t_stride,
+                        int32_t u_stride, int32_t D, int32_t activation,
+                        int32_t out_dtype, void *out, void *stream);
+
 /* ---- output projection of the joiner fused with the denominators (no
  * counterpart in the reference: its caller computes
  * logits = Linear(tanh(enc + dec)) with torch, README.md:166-177, and the loss

@@ -552,10 +552,16 @@ void check_joiner_inputs(const torch::Tensor &enc, const torch::Tensor &dec,
 // (packed (rows, D), row_splits (N+1) int32)
 std::pair<torch::Tensor, torch::Tensor> joiner_pack(
     const torch::Tensor &enc, const torch::Tensor &dec, const torch::Tensor &logit_lengths,
-    const torch::Tensor &target_lengths, const std::string &activation) {
+    const torch::Tensor &target_lengths, const std::string &activation,
+    const std::string &out_dtype) {
   const int act = activation_code(activation);
   check_joiner_inputs(enc, dec, logit_lengths, target_lengths);
   const int64_t N = enc.size(0), Tmax = enc.size(1), U1max = dec.size(1), D = enc.size(2);
+  const int odt = out_dtype == "float16" ? OT_DTYPE_F16 : out_dtype == "bfloat16" ? OT_DTYPE_BF16 : OT_DTYPE_F32;
+  TORCH_CHECK(odt != OT_DTYPE_F32 || out_dtype == "float32",
+              "pack_joiner: out_dtype must be float32, float16 or bfloat16, got ", out_dtype);
+  TORCH_CHECK(odt == OT_DTYPE_F32 || D % 8 == 0,
+              "pack_joiner: a 16-bit output needs D to be a multiple of 8, got ", D);
   c10::hip::HIPGuardMasqueradingAsCUDA device_guard(enc.device());
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
 
@@ -586,13 +592,24 @@ std::pair<torch::Tensor, torch::Tensor> joiner_pack(
   TORCH_CHECK(rows > 0 && rows <= INT32_MAX, "pack_joiner: sum of T * (U + 1) is ", rows,
               ", outside (0, 2^31)");
 
-  torch::Tensor out = torch::empty({rows, D}, enc.options());
+  torch::Tensor out = torch::empty(
+      {rows, D}, enc.options().dtype(odt == OT_DTYPE_F16    ? torch::kHalf
+                                     : odt == OT_DTYPE_BF16 ? torch::kBFloat16
+                                                            : torch::kFloat));
   {
     ScopedTimer timer("joiner_pack", stream);
-    OT_CHECK(ot_joiner_pack(enc.data_ptr<float>(), dec.data_ptr<float>(),
-                            logit_lengths.data_ptr<int32_t>(), target_lengths.data_ptr<int32_t>(),
-                            row_splits.data_ptr<int32_t>(), (int32_t)N, (int32_t)Tmax,
-                            (int32_t)U1max, (int32_t)D, act, out.data_ptr<float>(), stream));
+    if (odt == OT_DTYPE_F32) {
+      OT_CHECK(ot_joiner_pack(enc.data_ptr<float>(), dec.data_ptr<float>(),
+                              logit_lengths.data_ptr<int32_t>(), target_lengths.data_ptr<int32_t>(),
+                              row_splits.data_ptr<int32_t>(), (int32_t)N, (int32_t)Tmax,
+                              (int32_t)U1max, (int32_t)D, act, out.data_ptr<float>(), stream));
+    } else {
+      OT_CHECK(ot_joiner_pack_half(enc.data_ptr<float>(), dec.data_ptr<float>(),
+                                   logit_lengths.data_ptr<int32_t>(),
+                                   target_lengths.data_ptr<int32_t>(), row_splits.data_ptr<int32_t>(),
+                                   (int32_t)N, (int32_t)Tmax, (int32_t)U1max, (int32_t)D, act, odt,
+                                   out.data_ptr(), stream));
+    }
   }
   return {out, row_splits};
 }
@@ -703,6 +720,7 @@ PYBIND11_MODULE(_optimized_transducer, m) {
   m.def("scale_by_device_scalar_", &scale_by_device_scalar_, py::arg("x"), py::arg("factor"));
   m.def("joiner_pack", &joiner_pack, py::arg("encoder_out"), py::arg("decoder_out"),
         py::arg("logit_lengths"), py::arg("target_lengths"), py::arg("activation"),
+        py::arg("out_dtype") = "float32",
         "Packed joiner input act(enc[b,t] + dec[b,u]) for the valid (t, u) cells, in the row order "
         "of the loss; returns (packed (rows, D), row_splits).");
   m.def("joiner_unpack_grad", &joiner_unpack_grad, py::arg("grad_out"), py::arg("encoder_out"),

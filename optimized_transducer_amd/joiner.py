@@ -24,13 +24,15 @@ from . import _optimized_transducer
 
 class PackJoinerFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, encoder_out, decoder_out, logit_lengths, target_lengths, activation):
+    def forward(ctx, encoder_out, decoder_out, logit_lengths, target_lengths, activation,
+                out_dtype="float32"):
         out, row_splits = _optimized_transducer.joiner_pack(
             encoder_out=encoder_out,
             decoder_out=decoder_out,
             logit_lengths=logit_lengths,
             target_lengths=target_lengths,
             activation=activation,
+            out_dtype=out_dtype,
         )
         ctx.activation = activation
         ctx.save_for_backward(encoder_out, decoder_out, logit_lengths, target_lengths, row_splits)
@@ -39,8 +41,9 @@ class PackJoinerFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         encoder_out, decoder_out, logit_lengths, target_lengths, row_splits = ctx.saved_tensors
+        # the gradient pass is a float32 kernel: a 16-bit gradient is widened first
         grad_enc, grad_dec = _optimized_transducer.joiner_unpack_grad(
-            grad_out=grad_out.contiguous(),
+            grad_out=grad_out.float().contiguous(),
             encoder_out=encoder_out,
             decoder_out=decoder_out,
             logit_lengths=logit_lengths,
@@ -48,7 +51,7 @@ class PackJoinerFunction(torch.autograd.Function):
             row_splits=row_splits,
             activation=ctx.activation,
         )
-        return grad_enc, grad_dec, None, None, None
+        return grad_enc, grad_dec, None, None, None, None
 
 
 def pack_joiner(
@@ -57,6 +60,7 @@ def pack_joiner(
     logit_lengths: torch.Tensor,
     target_lengths: torch.Tensor,
     activation: Optional[str] = None,
+    out_dtype: torch.dtype = torch.float32,
 ) -> torch.Tensor:
     """Joiner input in the packed row order of :func:`transducer_loss`.
 
@@ -69,14 +73,21 @@ def pack_joiner(
       logit_lengths: (N,) int32, T_i (1 <= T_i <= T).
       target_lengths: (N,) int32, U_i (0 <= U_i <= U).
       activation: None / "none" for ``enc + dec``, "tanh" for ``tanh(enc + dec)``.
+      out_dtype: torch.float32, or torch.float16 / torch.bfloat16 (D a multiple of 8)
+        for a projection in 16 bits (:func:`project_joiner`): computed in float32 and
+        rounded once, without a float32 array and a cast pass in between.
     Returns:
-      (sum_i T_i * (U_i + 1), D) float32: row ``row_splits[i] + t * (U_i + 1) + u``
+      (sum_i T_i * (U_i + 1), D) of ``out_dtype``: row ``row_splits[i] + t * (U_i + 1) + u``
       holds ``act(encoder_out[i, t] + decoder_out[i, u])``.  Differentiable with
       respect to ``encoder_out`` and ``decoder_out`` (padding gets zero gradient).
     """
+    names = {torch.float32: "float32", torch.float16: "float16", torch.bfloat16: "bfloat16"}
+    if out_dtype not in names:
+        raise ValueError("pack_joiner: out_dtype must be torch.float32, torch.float16 or "
+                         "torch.bfloat16, got %r" % (out_dtype,))
     return PackJoinerFunction.apply(
         encoder_out, decoder_out, logit_lengths, target_lengths,
-        "none" if activation is None else activation,
+        "none" if activation is None else activation, names[out_dtype],
     )
 
 

@@ -251,3 +251,13 @@ def log_probs_given_den(logits, den, targets, U, splits, blank):
                                        ctypes.c_int64(rows), ctypes.c_int32(V), ctypes.c_int32(blank),
                                        ptr(lp), stream()))
     return lp
+
+
+def joiner_pack_half(enc, dec, T, U, splits, rows, activation, out_dtype):
+    N, Tm, D = enc.shape
+    out = torch.full((rows, D), float("nan"), dtype=out_dtype, device=enc.device)
+    check(lib().ot_joiner_pack_half(ptr(enc), ptr(dec), ptr(T), ptr(U), ptr(splits), ctypes.c_int32(N),
+                                    ctypes.c_int32(Tm), ctypes.c_int32(dec.shape[1]), ctypes.c_int32(D),
+                                    ctypes.c_int32(activation), ctypes.c_int32(DTYPE[out_dtype]), ptr(out),
+                                    stream()))
+    return out

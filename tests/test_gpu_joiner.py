@@ -160,3 +160,61 @@ def test_argument_checks(device):
     with pytest.raises(RuntimeError, match="logit_lengths >= 1"):
         ot.pack_joiner(de, dd, _dev(bad, device), dU)
     assert ot.pack_joiner(de, dd, dT, dU).shape == (int((T * (U + 1)).sum()), 8)
+
+
+HALF_CASES = [c for c in CASES if c[4] % 8 == 0]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("activation", [None, "tanh"])
+@pytest.mark.parametrize("case", HALF_CASES, ids=[c[0] for c in HALF_CASES])
+def test_pack_with_16_bit_output(case, activation, dtype, device):
+    """float32 arithmetic, one rounding to nearest even: the float32 kernel's output
+    rounded by torch gives the same bits."""
+    _, N, Tm, U1m, D, pad_t, pad_u = case
+    rng = np.random.default_rng(zlib.crc32(case[0].encode()) + 1)
+    T, U, enc, dec = _batch(rng, N, Tm, U1m, D, pad_t, pad_u)
+    dT, dU, denc, ddec = _dev(T, device), _dev(U, device), _dev(enc, device), _dev(dec, device)
+    splits, st = cabi.row_splits(dT, dU, torch.zeros((N, 0), dtype=torch.int32, device=device))
+    rows = int(st.sum_tu)
+    got = cabi.joiner_pack_half(denc, ddec, dT, dU, splits, rows, ACT[activation], dtype)
+    full = cabi.joiner_pack(denc, ddec, dT, dU, splits, rows, ACT[activation])
+    assert got.dtype == dtype and torch.equal(got, full.to(dtype))
+    want = torch.from_numpy(oracle.pack_joiner(enc, dec, T, U, activation)).to(dtype)
+    ulp = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    diff = (got.float().cpu() - want.float()).abs()
+    assert (diff <= 2 * ulp * want.float().abs() + 1e-6).all()
+
+
+def test_pack_16_bit_output_in_the_python_pipeline(device):
+    import optimized_transducer_amd as ot
+    rng = np.random.default_rng(8)
+    T, U, enc, dec = _batch(rng, 5, 14, 6, 64)
+    dT, dU = _dev(T, device), _dev(U, device)
+    te = _dev(enc, device).requires_grad_(True)
+    td = _dev(dec, device).requires_grad_(True)
+    x = ot.pack_joiner(te, td, dT, dU, activation="tanh", out_dtype=torch.bfloat16)
+    ref = ot.pack_joiner(te.detach(), td.detach(), dT, dU, activation="tanh")
+    assert x.dtype == torch.bfloat16 and torch.equal(x, ref.to(torch.bfloat16))
+    # joiner -> 16-bit projection with the denominators -> loss; gradients reach both inputs
+    torch.manual_seed(1)
+    w = (torch.randn(30, 64, device=device) / 8).to(torch.bfloat16).requires_grad_(True)
+    b = torch.randn(30, device=device, requires_grad=True)
+    tg = _dev(rng.integers(1, 30, size=(5, int(U.max()))).astype(np.int32), device)
+    logits, den = ot.project_joiner(x, w, b)
+    loss = ot.transducer_loss(logits, tg, dT, dU, 0, False, reduction="sum", denominators=den)
+    loss.backward()
+    # the same through float32 tensors and torch's own ops
+    re = _dev(enc, device).requires_grad_(True)
+    rd = _dev(dec, device).requires_grad_(True)
+    y = ot.pack_joiner(re, rd, dT, dU, activation="tanh")
+    l2 = ot.transducer_loss(torch.nn.functional.linear(y, w.detach().float(), b.detach()), tg, dT, dU, 0,
+                            False, reduction="sum")
+    l2.backward()
+    assert abs(loss.item() - l2.item()) <= 0.02 * abs(l2.item())
+    for a, r in ((te.grad, re.grad), (td.grad, rd.grad)):
+        assert (a - r).abs().max() <= 0.05 * r.abs().max() + 1e-4
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        ot.pack_joiner(torch.zeros(1, 2, 12, device=device), torch.zeros(1, 2, 12, device=device),
+                       torch.ones(1, dtype=torch.int32, device=device),
+                       torch.ones(1, dtype=torch.int32, device=device), out_dtype=torch.float16)
