@@ -315,6 +315,19 @@ int ot_joiner_pack_half(const float *enc, const float *dec,
                         int32_t u_stride, int32_t D, int32_t activation,
                         int32_t out_dtype, void *out, void *stream);
 
+/* ot_joiner_unpack_grad for an incoming gradient of grad_dtype (any of the
+ * three OT_DTYPE_*): a 16-bit gradient, as the backward of a 16-bit projection
+ * produces it, is widened on the fly; sums and outputs stay float32. */
+int ot_joiner_unpack_grad_from(const void *grad_out, int32_t grad_dtype,
+                               const float *enc, const float *dec,
+                               const int32_t *logit_lengths,
+                               const int32_t *target_lengths,
+                               const int32_t *row_splits, int32_t N,
+                               int32_t t_stride, int32_t u_stride, int32_t D,
+                               int32_t activation, void *workspace,
+                               size_t workspace_bytes, float *grad_enc,
+                               float *grad_dec, void *stream);
+
 /* ---- output projection of the joiner fused with the denominators (no
  * counterpart in the reference: its caller computes
  * logits = Linear(tanh(enc + dec)) with torch, README.md:166-177, and the loss

@@ -623,9 +623,9 @@ std::pair<torch::Tensor, torch::Tensor> joiner_unpack_grad(
   check_joiner_inputs(enc, dec, logit_lengths, target_lengths);
   const int64_t N = enc.size(0), Tmax = enc.size(1), U1max = dec.size(1), D = enc.size(2);
   TORCH_CHECK(grad_out.is_cuda() && grad_out.device() == enc.device() &&
-                  grad_out.scalar_type() == torch::kFloat && grad_out.dim() == 2 &&
-                  grad_out.size(1) == D && grad_out.is_contiguous(),
-              "pack_joiner backward: the gradient must be a contiguous float32 (rows, ", D,
+                  (grad_out.scalar_type() == torch::kFloat || half_dtype(grad_out) != OT_DTYPE_F32) &&
+                  grad_out.dim() == 2 && grad_out.size(1) == D && grad_out.is_contiguous(),
+              "pack_joiner backward: the gradient must be a contiguous float32, float16 or bfloat16 (rows, ", D,
               ") tensor on the device of encoder_out");
   TORCH_CHECK(row_splits.is_cuda() && row_splits.device() == enc.device() &&
                   row_splits.scalar_type() == torch::kInt32 && row_splits.dim() == 1 &&
@@ -639,7 +639,7 @@ std::pair<torch::Tensor, torch::Tensor> joiner_unpack_grad(
   torch::Tensor grad_enc = torch::empty_like(enc);
   torch::Tensor grad_dec = torch::empty_like(dec);
   ScopedTimer timer("joiner_unpack_grad", stream);
-  OT_CHECK(ot_joiner_unpack_grad(grad_out.data_ptr<float>(), enc.data_ptr<float>(),
+  OT_CHECK(ot_joiner_unpack_grad_from(grad_out.data_ptr(), half_dtype(grad_out), enc.data_ptr<float>(),
                                  dec.data_ptr<float>(), logit_lengths.data_ptr<int32_t>(),
                                  target_lengths.data_ptr<int32_t>(), row_splits.data_ptr<int32_t>(),
                                  (int32_t)N, (int32_t)Tmax, (int32_t)U1max, (int32_t)D, act,

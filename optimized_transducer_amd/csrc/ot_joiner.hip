@@ -186,8 +186,8 @@ __global__ __launch_bounds__(kBlock) void joiner_pack_half_kernel(
 // backward
 // ---------------------------------------------------------------------------
 constexpr int kTileFrames = OT_JOINER_TILE_FRAMES;  // frames per workgroup
-constexpr int kSlabLanes = 16;                      // lanes across the columns of a slab
-constexpr int kUPhases = kBlock / kSlabLanes;       // positions u in flight per workgroup
+constexpr int kSlabLanes = 16;      // lanes across the columns of a slab: 16 x 16 bytes of a float32 row,
+constexpr int kSlabLanesHalf = 32;  // 32 x 8 bytes of a 2-byte row (256 contiguous bytes either way)
 
 // One workgroup: utterance b = blockIdx.z, frames [t0, t0 + 16), columns
 // [slab*16*VEC, (slab+1)*16*VEC).  Thread (phase, lane): columns lane*VEC.., and
@@ -195,20 +195,52 @@ constexpr int kUPhases = kBlock / kSlabLanes;       // positions u in flight per
 // values (16 independent loads), adds them up for the decoder and into 16
 // per-frame accumulators for the encoder.  The encoder sums of the workgroup's
 // threads are then added through DPP/LDS in a fixed order.
-template <int VEC, int ACT>
+// VEC elements of the incoming gradient: float32 (G = float) or a 2-byte type.  Loading
+// and widening are two steps so that a thread's 16 loads are all issued before the
+// first value is used.
+template <class G, int VEC> struct GradIO {
+  typedef unsigned short raw_t __attribute__((ext_vector_type(VEC == 4 ? 4 : 2)));
+  static __device__ __forceinline__ raw_t load(const void *base, int64_t index) {
+    const unsigned short *p = static_cast<const unsigned short *>(base) + index;
+    raw_t r;
+    if (VEC == 4) {
+      r = *reinterpret_cast<const raw_t *>(p);
+    } else {
+      r[0] = *p;
+      r[1] = 0;
+    }
+    return r;
+  }
+  static __device__ __forceinline__ void widen(raw_t r, Vec<VEC> &g) {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) g.v[k] = to_float<G>(r[k]);
+  }
+};
+template <int VEC> struct GradIO<float, VEC> {
+  typedef Vec<VEC> raw_t;
+  static __device__ __forceinline__ raw_t load(const void *base, int64_t index) {
+    raw_t r;
+    r.load(static_cast<const float *>(base) + index);
+    return r;
+  }
+  static __device__ __forceinline__ void widen(const raw_t &r, Vec<VEC> &g) { g = r; }
+};
+
+// G: element type of grad_out (float, F16 or BF16); everything else is float32.
+template <int VEC, int ACT, class G, int SL>
 __global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
-    const float *__restrict__ grad_out, const float *__restrict__ enc,
+    const void *__restrict__ grad_out, const float *__restrict__ enc,
     const float *__restrict__ dec, const int32_t *__restrict__ logit_lengths,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
     int t_stride, int u_stride, int D, float *__restrict__ grad_enc,
     float *__restrict__ dec_partial) {
-  __shared__ __attribute__((aligned(16))) float s_enc[kTileFrames][kSlabLanes * VEC];
-  __shared__ __attribute__((aligned(16))) float s_red[kWavesPerBlock][kTileFrames][kSlabLanes * VEC];
+  __shared__ __attribute__((aligned(16))) float s_enc[kTileFrames][SL * VEC];
+  __shared__ __attribute__((aligned(16))) float s_red[kWavesPerBlock][kTileFrames][SL * VEC];
   const int b = blockIdx.z;
   const int t0 = blockIdx.y * kTileFrames;
-  const int lane = threadIdx.x & (kSlabLanes - 1);
-  const int phase = threadIdx.x / kSlabLanes;
-  const int col = (blockIdx.x * kSlabLanes + lane) * VEC;
+  const int lane = threadIdx.x & (SL - 1);
+  const int phase = threadIdx.x / SL;
+  const int col = (blockIdx.x * SL + lane) * VEC;
   const bool col_ok = col < D;  // D is a multiple of VEC
   const int T = min(logit_lengths[b], t_stride);
   const int U1 = min(target_lengths[b] + 1, u_stride);
@@ -219,7 +251,7 @@ __global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
   // output) gets zeros
   const int nframes = max(0, min(kTileFrames, T - t0));
   if (ACT != OT_ACT_NONE) {
-    for (int i = phase; i < kTileFrames; i += kUPhases) {
+    for (int i = phase; i < kTileFrames; i += (kBlock / SL)) {
       Vec<VEC> e;
 #pragma unroll
       for (int k = 0; k < VEC; ++k) e.v[k] = 0.f;
@@ -237,14 +269,19 @@ __global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
 
   if (nframes > 0 && col_ok) {
     const int64_t frame_stride = (int64_t)U1 * D;
-    for (int u = phase; u < U1; u += kUPhases) {
-      const float *p = grad_out + ((row0 + (int64_t)t0 * U1 + u) * D + col);
+    for (int u = phase; u < U1; u += (kBlock / SL)) {
+      const int64_t p = (row0 + (int64_t)t0 * U1 + u) * D + col;
+      // frames past the tile's last one re-read frame 0 and are zeroed afterwards: no
+      // branch between the loads
+      typename GradIO<G, VEC>::raw_t raw[kTileFrames];
+#pragma unroll
+      for (int i = 0; i < kTileFrames; ++i)
+        raw[i] = GradIO<G, VEC>::load(grad_out, p + (i < nframes ? i : 0) * frame_stride);
       Vec<VEC> g[kTileFrames];
 #pragma unroll
       for (int i = 0; i < kTileFrames; ++i) {
-        if (i < nframes) {
-          g[i].load(p + i * frame_stride);
-        } else {
+        GradIO<G, VEC>::widen(raw[i], g[i]);
+        if (i >= nframes) {
 #pragma unroll
           for (int k = 0; k < VEC; ++k) g[i].v[k] = 0.f;
         }
@@ -277,20 +314,20 @@ __global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
 #pragma unroll
     for (int k = 0; k < VEC; ++k) {
       float v = acc[i].v[k];
-      if (kSlabLanes <= 16) v += __shfl_xor(v, 16, kWave);
-      if (kSlabLanes <= 32) v += __shfl_xor(v, 32, kWave);
+      if (SL <= 16) v += __shfl_xor(v, 16, kWave);
+      if (SL <= 32) v += __shfl_xor(v, 32, kWave);
       acc[i].v[k] = v;
     }
   const int wave = threadIdx.x / kWave;
-  if ((threadIdx.x & (kWave - 1)) < kSlabLanes) {
+  if ((threadIdx.x & (kWave - 1)) < SL) {
 #pragma unroll
     for (int i = 0; i < kTileFrames; ++i) acc[i].store_lds(&s_red[wave][i][lane * VEC]);
   }
   __syncthreads();
-  // 16 frames x kSlabLanes (frame, lane) pairs over the workgroup's threads
-  for (int pair = threadIdx.x; pair < kTileFrames * kSlabLanes; pair += kBlock) {
-    const int i = pair / kSlabLanes, l = pair & (kSlabLanes - 1);
-    const int c = (blockIdx.x * kSlabLanes + l) * VEC;
+  // 16 frames x SL (frame, lane) pairs over the workgroup's threads
+  for (int pair = threadIdx.x; pair < kTileFrames * SL; pair += kBlock) {
+    const int i = pair / SL, l = pair & (SL - 1);
+    const int c = (blockIdx.x * SL + l) * VEC;
     const int t = t0 + i;
     if (t < t_stride && c < D) {
       Vec<VEC> r;
@@ -413,11 +450,15 @@ size_t ot_joiner_unpack_workspace_bytes(int32_t N, int32_t t_stride, int32_t u_s
   return (size_t)N * ntiles * (size_t)u_stride * (size_t)D * sizeof(float);
 }
 
-int ot_joiner_unpack_grad(const float *grad_out, const float *enc, const float *dec,
-                          const int32_t *logit_lengths, const int32_t *target_lengths,
-                          const int32_t *row_splits, int32_t N, int32_t t_stride, int32_t u_stride,
-                          int32_t D, int32_t activation, void *workspace, size_t workspace_bytes,
-                          float *grad_enc, float *grad_dec, void *stream) {
+int ot_joiner_unpack_grad_from(const void *grad_out, int32_t grad_dtype, const float *enc,
+                               const float *dec, const int32_t *logit_lengths,
+                               const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
+                               int32_t t_stride, int32_t u_stride, int32_t D, int32_t activation,
+                               void *workspace, size_t workspace_bytes, float *grad_enc,
+                               float *grad_dec, void *stream) {
+  if (grad_dtype != OT_DTYPE_F32 && grad_dtype != OT_DTYPE_F16 && grad_dtype != OT_DTYPE_BF16)
+    return OT_E_BAD_ARG;
+  const bool g32 = grad_dtype == OT_DTYPE_F32;
   if (!grad_out || !logit_lengths || !target_lengths || !row_splits || !workspace || !grad_enc ||
       !grad_dec || N <= 0 || N > 65535 || t_stride <= 0 || u_stride <= 0 || D <= 0 ||
       (int64_t)N * t_stride > INT32_MAX || (int64_t)N * u_stride > INT32_MAX ||
@@ -426,27 +467,34 @@ int ot_joiner_unpack_grad(const float *grad_out, const float *enc, const float *
     return OT_E_BAD_ARG;
   if (workspace_bytes < ot_joiner_unpack_workspace_bytes(N, t_stride, u_stride, D))
     return OT_E_BAD_ARG;
-  if (!aligned4(grad_out) || !aligned4(enc) || !aligned4(dec) || !aligned4(grad_enc) ||
-      !aligned4(grad_dec) || !aligned16(workspace))
+  if ((reinterpret_cast<uintptr_t>(grad_out) & (g32 ? 3 : 1)) || !aligned4(enc) || !aligned4(dec) ||
+      !aligned4(grad_enc) || !aligned4(grad_dec) || !aligned16(workspace))
     return OT_E_MISALIGNED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool v4 = D % 4 == 0 && aligned16(grad_out) && aligned16(grad_enc) && aligned16(grad_dec) &&
+  // 4 columns per thread need 16-byte (float32) / 8-byte (2-byte types) aligned rows
+  const bool v4 = D % 4 == 0 && (reinterpret_cast<uintptr_t>(grad_out) & (g32 ? 15 : 7)) == 0 &&
+                  aligned16(grad_enc) && aligned16(grad_dec) &&
                   (activation == OT_ACT_NONE || (aligned16(enc) && aligned16(dec)));
   const int vec = v4 ? 4 : 1;
   const int ntiles = (t_stride + kTileFrames - 1) / kTileFrames;
   if (ntiles > 65535) return OT_E_TOO_LONG;
-  const int slab = kSlabLanes * vec;
+  const int slab = (g32 ? kSlabLanes : kSlabLanesHalf) * vec;
   const dim3 grid((unsigned)((D + slab - 1) / slab), (unsigned)ntiles, (unsigned)N);
   float *partial = static_cast<float *>(workspace);
-#define OT_LAUNCH_UNPACK(VEC_, ACT_)                                                          \
-  hipLaunchKernelGGL((joiner_unpack_grad_kernel<VEC_, ACT_>), grid, dim3(kBlock), 0, s,       \
+#define OT_LAUNCH_UNPACK(VEC_, ACT_, G_, SL_)                                                 \
+  hipLaunchKernelGGL((joiner_unpack_grad_kernel<VEC_, ACT_, G_, SL_>), grid, dim3(kBlock), 0, s, \
                      grad_out, enc, dec, logit_lengths, target_lengths, row_splits, t_stride, \
                      u_stride, D, grad_enc, partial)
+#define OT_LAUNCH_UNPACK_G(VEC_, ACT_)                                                  \
+  if (g32) OT_LAUNCH_UNPACK(VEC_, ACT_, float, kSlabLanes);                             \
+  else if (grad_dtype == OT_DTYPE_F16) OT_LAUNCH_UNPACK(VEC_, ACT_, F16, kSlabLanesHalf); \
+  else OT_LAUNCH_UNPACK(VEC_, ACT_, BF16, kSlabLanesHalf)
   if (activation == OT_ACT_TANH) {
-    if (vec == 4) OT_LAUNCH_UNPACK(4, OT_ACT_TANH); else OT_LAUNCH_UNPACK(1, OT_ACT_TANH);
+    if (vec == 4) { OT_LAUNCH_UNPACK_G(4, OT_ACT_TANH); } else { OT_LAUNCH_UNPACK_G(1, OT_ACT_TANH); }
   } else {
-    if (vec == 4) OT_LAUNCH_UNPACK(4, OT_ACT_NONE); else OT_LAUNCH_UNPACK(1, OT_ACT_NONE);
+    if (vec == 4) { OT_LAUNCH_UNPACK_G(4, OT_ACT_NONE); } else { OT_LAUNCH_UNPACK_G(1, OT_ACT_NONE); }
   }
+#undef OT_LAUNCH_UNPACK_G
 #undef OT_LAUNCH_UNPACK
   int rc = launch_status();
   if (rc) return rc;
@@ -462,6 +510,16 @@ int ot_joiner_unpack_grad(const float *grad_out, const float *enc, const float *
                        partial, logit_lengths, target_lengths, N, t_stride, u_stride, D, ntiles,
                        grad_dec);
   return launch_status();
+}
+
+int ot_joiner_unpack_grad(const float *grad_out, const float *enc, const float *dec,
+                          const int32_t *logit_lengths, const int32_t *target_lengths,
+                          const int32_t *row_splits, int32_t N, int32_t t_stride, int32_t u_stride,
+                          int32_t D, int32_t activation, void *workspace, size_t workspace_bytes,
+                          float *grad_enc, float *grad_dec, void *stream) {
+  return ot_joiner_unpack_grad_from(grad_out, OT_DTYPE_F32, enc, dec, logit_lengths, target_lengths,
+                                    row_splits, N, t_stride, u_stride, D, activation, workspace,
+                                    workspace_bytes, grad_enc, grad_dec, stream);
 }
 
 }  // extern "C"

@@ -41,9 +41,11 @@ class PackJoinerFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         encoder_out, decoder_out, logit_lengths, target_lengths, row_splits = ctx.saved_tensors
-        # the gradient pass is a float32 kernel: a 16-bit gradient is widened first
+        # float32, float16 or bfloat16: a 16-bit gradient is widened inside the kernel
+        if grad_out.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+            grad_out = grad_out.float()
         grad_enc, grad_dec = _optimized_transducer.joiner_unpack_grad(
-            grad_out=grad_out.float().contiguous(),
+            grad_out=grad_out.contiguous(),
             encoder_out=encoder_out,
             decoder_out=decoder_out,
             logit_lengths=logit_lengths,

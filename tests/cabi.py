@@ -173,11 +173,19 @@ def joiner_unpack_grad(grad_out, enc, dec, T, U, splits, activation):
     ws = torch.empty(nbytes, dtype=torch.uint8, device=enc.device)
     ge = torch.full_like(enc, float("nan"))
     gd = torch.full_like(dec, float("nan"))
-    check(L.ot_joiner_unpack_grad(ptr(grad_out), ptr(enc), ptr(dec), ptr(T), ptr(U), ptr(splits),
-                                  ctypes.c_int32(N), ctypes.c_int32(t_stride),
-                                  ctypes.c_int32(u_stride), ctypes.c_int32(D),
-                                  ctypes.c_int32(activation), ptr(ws), ctypes.c_size_t(nbytes),
-                                  ptr(ge), ptr(gd), stream()))
+    if grad_out.dtype == torch.float32:
+        check(L.ot_joiner_unpack_grad(ptr(grad_out), ptr(enc), ptr(dec), ptr(T), ptr(U), ptr(splits),
+                                      ctypes.c_int32(N), ctypes.c_int32(t_stride),
+                                      ctypes.c_int32(u_stride), ctypes.c_int32(D),
+                                      ctypes.c_int32(activation), ptr(ws), ctypes.c_size_t(nbytes),
+                                      ptr(ge), ptr(gd), stream()))
+    else:  # a 16-bit incoming gradient
+        code = {torch.float16: 1, torch.bfloat16: 2}[grad_out.dtype]
+        check(L.ot_joiner_unpack_grad_from(ptr(grad_out), ctypes.c_int32(code), ptr(enc), ptr(dec),
+                                           ptr(T), ptr(U), ptr(splits), ctypes.c_int32(N),
+                                           ctypes.c_int32(t_stride), ctypes.c_int32(u_stride),
+                                           ctypes.c_int32(D), ctypes.c_int32(activation), ptr(ws),
+                                           ctypes.c_size_t(nbytes), ptr(ge), ptr(gd), stream()))
     return ge, gd
 
 

@@ -218,3 +218,28 @@ def test_pack_16_bit_output_in_the_python_pipeline(device):
         ot.pack_joiner(torch.zeros(1, 2, 12, device=device), torch.zeros(1, 2, 12, device=device),
                        torch.ones(1, dtype=torch.int32, device=device),
                        torch.ones(1, dtype=torch.int32, device=device), out_dtype=torch.float16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("activation", [None, "tanh"])
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_unpack_of_a_16_bit_gradient(case, activation, dtype, device):
+    """The incoming gradient is widened (exactly) inside the kernel, for 4 columns per thread and
+    for the scalar path; the sums are taken in another order than in the float32 kernel (wider
+    slabs), so the oracle's bound applies, not bit equality."""
+    _, N, Tm, U1m, D, pad_t, pad_u = case
+    rng = np.random.default_rng(zlib.crc32(case[0].encode()) + 2)
+    T, U, enc, dec = _batch(rng, N, Tm, U1m, D, pad_t, pad_u)
+    dT, dU, denc, ddec = _dev(T, device), _dev(U, device), _dev(enc, device), _dev(dec, device)
+    splits, st = cabi.row_splits(dT, dU, torch.zeros((N, 0), dtype=torch.int32, device=device))
+    g = torch.from_numpy(rng.standard_normal((int(st.sum_tu), D)).astype(np.float32)).to(dtype).to(device)
+    ge, gd = cabi.joiner_unpack_grad(g, denc, ddec, dT, dU, splits, ACT[activation])
+    ge, gd = ge.cpu().numpy(), gd.cpu().numpy()
+    we, wd, ae, ad = oracle.pack_joiner_backward(g.float().cpu().numpy(), enc, dec, T, U, activation)
+    assert not np.isnan(ge).any() and not np.isnan(gd).any()
+    assert (np.abs(ge - we) <= 1e-5 * np.abs(we) + 1e-6 * ae + 1e-30).all(), np.abs(ge - we).max()
+    assert (np.abs(gd - wd) <= 1e-5 * np.abs(wd) + 1e-6 * ad + 1e-30).all(), np.abs(gd - wd).max()
+    for b in range(N):  # padding is exactly zero
+        assert (ge[b, T[b]:] == 0).all() and (gd[b, U[b] + 1:] == 0).all()
+    ge2, gd2 = cabi.joiner_unpack_grad(g, denc, ddec, dT, dU, splits, ACT[activation])
+    assert (ge2.cpu().numpy() == ge).all() and (gd2.cpu().numpy() == gd).all()  # fixed order
