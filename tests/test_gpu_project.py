@@ -49,7 +49,9 @@ def _check(x, w, b, out_dtype):
 @pytest.mark.parametrize("rows,D,V", [(700, 64, 500), (256, 64, 128), (1, 512, 37), (513, 192, 1030),
                                       (300, 128, 6), (64, 256, 130),
                                       # more 128-row tiles than resident workgroups: some take two
-                                      (70001, 64, 40), (66000, 64, 300)])
+                                      (70001, 64, 40), (66000, 64, 300),
+                                      # many passes over the vocabulary, long rows of x
+                                      (300, 128, 5000), (200, 1024, 777)])
 def test_projection_and_denominators(rows, D, V, dtype, out, device):
     rng = np.random.default_rng(rows * 7 + V)
     dt = HALF[dtype]
