@@ -119,7 +119,8 @@ def test_lattice_kernel_given_oracle_log_probs(case, device):
     assert (a2.cpu().numpy() == a).all() and (b2.cpu().numpy() == b).all()
 
 
-WIDE = [  # (T, U) per utterance: 3..16 waves per workgroup, mixed with short targets
+WIDE = [  # (T, U) per utterance: 2..16 waves' worth of columns, mixed with short targets
+    ("two_waves", [(50, 127), (9, 64), (20, 5), (1, 100), (70, 65), (33, 126)]),
     ("three_waves", [(50, 130), (9, 191), (20, 5)]),
     ("four_waves", [(300, 200), (7, 255), (64, 64), (1, 250)]),
     ("five_waves", [(40, 300), (3, 319), (100, 0)]),
