@@ -169,8 +169,9 @@ HALF_CASES = [c for c in CASES if c[4] % 8 == 0]
 @pytest.mark.parametrize("activation", [None, "tanh"])
 @pytest.mark.parametrize("case", HALF_CASES, ids=[c[0] for c in HALF_CASES])
 def test_pack_with_16_bit_output(case, activation, dtype, device):
-    """float32 arithmetic, one rounding to nearest even: the float32 kernel's output
-    rounded by torch gives the same bits."""
+    """float32 arithmetic, one rounding to nearest even: without activation the float32
+    kernel's output rounded by torch gives the same bits; the tanh of this kernel is accurate
+    to the 16-bit result, so it may differ from that by one unit in the last place."""
     _, N, Tm, U1m, D, pad_t, pad_u = case
     rng = np.random.default_rng(zlib.crc32(case[0].encode()) + 1)
     T, U, enc, dec = _batch(rng, N, Tm, U1m, D, pad_t, pad_u)
@@ -179,7 +180,14 @@ def test_pack_with_16_bit_output(case, activation, dtype, device):
     rows = int(st.sum_tu)
     got = cabi.joiner_pack_half(denc, ddec, dT, dU, splits, rows, ACT[activation], dtype)
     full = cabi.joiner_pack(denc, ddec, dT, dU, splits, rows, ACT[activation])
-    assert got.dtype == dtype and torch.equal(got, full.to(dtype))
+    assert got.dtype == dtype
+    if activation is None:
+        assert torch.equal(got, full.to(dtype))
+    else:
+        one = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7   # one unit in the last place
+        d = (got.float() - full.to(dtype).float()).abs()
+        assert (d <= one * full.abs() + 1e-7).all()
+        assert (d > 0).float().mean() < 0.02   # and rarely differs at all
     want = torch.from_numpy(oracle.pack_joiner(enc, dec, T, U, activation)).to(dtype)
     ulp = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
     diff = (got.float().cpu() - want.float()).abs()
@@ -195,7 +203,8 @@ def test_pack_16_bit_output_in_the_python_pipeline(device):
     td = _dev(dec, device).requires_grad_(True)
     x = ot.pack_joiner(te, td, dT, dU, activation="tanh", out_dtype=torch.bfloat16)
     ref = ot.pack_joiner(te.detach(), td.detach(), dT, dU, activation="tanh")
-    assert x.dtype == torch.bfloat16 and torch.equal(x, ref.to(torch.bfloat16))
+    assert x.dtype == torch.bfloat16
+    assert ((x.float() - ref).abs() <= 2.0 ** -7 * ref.abs() + 1e-7).all()
     # joiner -> 16-bit projection with the denominators -> loss; gradients reach both inputs
     torch.manual_seed(1)
     w = (torch.randn(30, 64, device=device) / 8).to(torch.bfloat16).requires_grad_(True)
