@@ -106,6 +106,20 @@ int ot_alpha_beta(const float *lp, const int32_t *logit_lengths,
                   float *alpha, float *beta, float *scores_alpha,
                   float *scores_beta, void *stream);
 
+/* ot_alpha_beta for a caller that has not validated the batch yet (the host
+ * is still waiting for ot_row_splits' status): every workgroup first checks on
+ * the device that row_splits[N] == rows, T_b >= 1, U_b >= 0 and that the
+ * utterance's cells fit 32-bit offsets, and writes nothing otherwise, so the
+ * launch is memory-safe for any lengths; max_u1 may be an upper bound
+ * (targets_cols + 1).  Results are meaningful only if the caller's own checks
+ * pass afterwards. */
+int ot_alpha_beta_guarded(const float *lp, const int32_t *logit_lengths,
+                          const int32_t *target_lengths,
+                          const int32_t *row_splits, int32_t N, int32_t max_u1,
+                          int32_t one_sym_per_frame, int64_t rows, float *alpha,
+                          float *beta, float *scores_alpha, float *scores_beta,
+                          void *stream);
+
 /* ot_alpha_beta restricted to utterances [utt_begin, utt_end); all arrays keep
  * their full-batch indexing. */
 int ot_alpha_beta_range(const float *lp, const int32_t *logit_lengths,

@@ -311,6 +311,19 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
       OT_CHECK_HIP(hipEventRecord(lse_b_done.ev, stream));
     }
   }
+  // The lattice kernel goes out before the host wait as well: it writes workspace
+  // only and checks on the device what its memory safety rests on, with
+  // targets.size(1) + 1 columns (what target_lengths.max() + 1 must be, checked below).
+  // The host's wake-up and its remaining launches then hide behind it even when the
+  // first kernel is the short gather of log-softmax input.
+  torch::Tensor scores = torch::empty({N}, logits.options().dtype(torch::kFloat));
+  const bool early_lattice = blank_ok && !overlap && S + 1 <= OT_MAX_U1;
+  if (early_lattice) {
+    ScopedTimer timer("alpha_beta", stream);
+    OT_CHECK(ot_alpha_beta_guarded(lp, p_T, p_U, row_splits, (int32_t)N, (int32_t)S + 1,
+                                   one_sym_per_frame, rows, alpha, beta, scores.data_ptr<float>(),
+                                   scores_beta, stream));
+  }
   OT_CHECK_HIP(hipEventSynchronize(status_ready.ev));
   const ot_batch_status st = *reinterpret_cast<const ot_batch_status *>(status_host.data_ptr());
   const int32_t *splits_host = reinterpret_cast<const int32_t *>(
@@ -332,7 +345,6 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
               "an utterance with T = ", st.logit_len_max, " and up to ", max_u1,
               " lattice columns is too large for the lattice kernel");
 
-  torch::Tensor scores = torch::empty({N}, logits.options().dtype(torch::kFloat));
   torch::Tensor gradient;
   const bool want_grad = logits.requires_grad();
   if (want_grad && !defer) {
@@ -344,7 +356,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
 
   // lattice + per-row coefficients of utterances [b0, b1) on stream `s`
   auto lattice_part = [&](int32_t b0, int32_t b1, hipStream_t s) {
-    {
+    if (!early_lattice) {
       ScopedTimer timer("alpha_beta", s);
       OT_CHECK(ot_alpha_beta_range(lp, p_T, p_U, row_splits, (int32_t)N, max_u1,
                                    one_sym_per_frame, b0, b1, alpha, beta,

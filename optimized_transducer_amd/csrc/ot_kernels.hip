@@ -572,16 +572,30 @@ __device__ __forceinline__ void lattice_sweep_staged(const float *__restrict__ l
   }
 }
 
+// A lattice kernel that is launched before the host has seen the batch facts checks
+// what its memory safety rests on itself and does nothing otherwise (guard_n = N, or 0
+// for a launch after validation): the rows of the batch add up to the size of the
+// arrays, every utterance has T >= 1 and 0 <= U < the workgroup's columns, and its cells
+// fit 32-bit byte offsets.
+__device__ __forceinline__ bool lattice_guard_ok(const int32_t *__restrict__ row_splits, int guard_n,
+                                                 int64_t guard_rows, int T, int U) {
+  if (guard_n <= 0) return true;
+  return (int64_t)row_splits[guard_n] == guard_rows && T >= 1 && U >= 0 && U < (int)blockDim.x &&
+         ((int64_t)T + 1300) * ((int64_t)U + 1) < ((int64_t)1 << 29);
+}
+
 template <int G, int THREADS>
 __global__ __launch_bounds__(THREADS) void alpha_beta_staged_kernel(
     const float *__restrict__ lp, const int32_t *__restrict__ logit_lengths,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
     int utt_begin, float *__restrict__ alpha, float *__restrict__ beta,
-    float *__restrict__ scores_alpha, float *__restrict__ scores_beta) {
+    float *__restrict__ scores_alpha, float *__restrict__ scores_beta, int guard_n,
+    int64_t guard_rows) {
   __shared__ float s_ring[THREADS / kWave][kRing + kChunk];
   extern __shared__ __attribute__((aligned(16))) float s_stage[];
   const int b = utt_begin + blockIdx.x;
   const int T = logit_lengths[b], U = target_lengths[b];
+  if (!lattice_guard_ok(row_splits, guard_n, guard_rows, T, U)) return;
   const int64_t row0 = row_splits[b];
   if (blockIdx.y == 0)
     lattice_sweep_staged<false, G>(lp, T, U, row0, alpha, scores_alpha + b, s_ring, s_stage);
@@ -594,10 +608,12 @@ __global__ __launch_bounds__(OT_MAX_U1) void alpha_beta_kernel(
     const float *__restrict__ lp, const int32_t *__restrict__ logit_lengths,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
     int utt_begin, float *__restrict__ alpha, float *__restrict__ beta,
-    float *__restrict__ scores_alpha, float *__restrict__ scores_beta) {
+    float *__restrict__ scores_alpha, float *__restrict__ scores_beta, int guard_n,
+    int64_t guard_rows) {
   __shared__ float s_ring[MULTI ? kMaxDpWaves : 1][kRing + kChunk];
   const int b = utt_begin + blockIdx.x;
   const int T = logit_lengths[b], U = target_lengths[b];
+  if (!lattice_guard_ok(row_splits, guard_n, guard_rows, T, U)) return;
   const int64_t row0 = row_splits[b];
   if (blockIdx.y == 0)
     lattice_sweep<false, OSF, MULTI>(lp, T, U, row0, alpha, scores_alpha + b, s_ring);
@@ -936,11 +952,11 @@ int ot_log_probs(const float *logits, const int32_t *targets, const int32_t *tar
                             blank, from_log_softmax, 0, rows, den, lp, stream);
 }
 
-int ot_alpha_beta_range(const float *lp, const int32_t *logit_lengths,
-                        const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
-                        int32_t max_u1, int32_t one_sym_per_frame, int32_t utt_begin,
-                        int32_t utt_end, float *alpha, float *beta, float *scores_alpha,
-                        float *scores_beta, void *stream) {
+static int launch_alpha_beta(const float *lp, const int32_t *logit_lengths,
+                             const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
+                             int32_t max_u1, int32_t one_sym_per_frame, int32_t utt_begin,
+                             int32_t utt_end, float *alpha, float *beta, float *scores_alpha,
+                             float *scores_beta, int guard_n, int64_t guard_rows, void *stream) {
   if (!lp || !logit_lengths || !target_lengths || !row_splits || !alpha || !beta ||
       !scores_alpha || !scores_beta || N <= 0 || max_u1 <= 0 || utt_begin < 0 || utt_end > N ||
       utt_begin > utt_end)
@@ -959,7 +975,7 @@ int ot_alpha_beta_range(const float *lp, const int32_t *logit_lengths,
 #define OT_LAUNCH_DPS(G_, THREADS_)                                                             \
   hipLaunchKernelGGL((alpha_beta_staged_kernel<G_, THREADS_>), grid, block, lds, s, lp,         \
                      logit_lengths, target_lengths, row_splits, utt_begin, alpha, beta,         \
-                     scores_alpha, scores_beta)
+                     scores_alpha, scores_beta, guard_n, guard_rows)
     if (G == 16) OT_LAUNCH_DPS(16, 256);
     else if (G == 8) OT_LAUNCH_DPS(8, 576);
     else OT_LAUNCH_DPS(4, 1024);
@@ -968,7 +984,8 @@ int ot_alpha_beta_range(const float *lp, const int32_t *logit_lengths,
   }
 #define OT_LAUNCH_DP(OSF_, MULTI_)                                                              \
   hipLaunchKernelGGL((alpha_beta_kernel<OSF_, MULTI_>), grid, block, 0, s, lp, logit_lengths,   \
-                     target_lengths, row_splits, utt_begin, alpha, beta, scores_alpha, scores_beta)
+                     target_lengths, row_splits, utt_begin, alpha, beta, scores_alpha, scores_beta, \
+                     guard_n, guard_rows)
   if (one_sym_per_frame) {
     if (multi) OT_LAUNCH_DP(true, true); else OT_LAUNCH_DP(true, false);
   } else {
@@ -976,6 +993,26 @@ int ot_alpha_beta_range(const float *lp, const int32_t *logit_lengths,
   }
 #undef OT_LAUNCH_DP
   return launch_status();
+}
+
+int ot_alpha_beta_range(const float *lp, const int32_t *logit_lengths,
+                        const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
+                        int32_t max_u1, int32_t one_sym_per_frame, int32_t utt_begin,
+                        int32_t utt_end, float *alpha, float *beta, float *scores_alpha,
+                        float *scores_beta, void *stream) {
+  return launch_alpha_beta(lp, logit_lengths, target_lengths, row_splits, N, max_u1,
+                           one_sym_per_frame, utt_begin, utt_end, alpha, beta, scores_alpha,
+                           scores_beta, 0, 0, stream);
+}
+
+int ot_alpha_beta_guarded(const float *lp, const int32_t *logit_lengths,
+                          const int32_t *target_lengths, const int32_t *row_splits, int32_t N,
+                          int32_t max_u1, int32_t one_sym_per_frame, int64_t rows, float *alpha,
+                          float *beta, float *scores_alpha, float *scores_beta, void *stream) {
+  if (rows <= 0) return OT_E_BAD_ARG;
+  return launch_alpha_beta(lp, logit_lengths, target_lengths, row_splits, N, max_u1,
+                           one_sym_per_frame, 0, N, alpha, beta, scores_alpha, scores_beta, N, rows,
+                           stream);
 }
 
 int ot_alpha_beta(const float *lp, const int32_t *logit_lengths, const int32_t *target_lengths,
