@@ -87,6 +87,21 @@ def alpha_beta(lp, T, U, splits, max_u1, one_sym_per_frame):
     return alpha, beta, sa, sb
 
 
+def alpha_beta_guarded(lp, T, U, splits, max_u1, one_sym_per_frame, rows):
+    """ot_alpha_beta_guarded: `rows` is what the caller believes the batch adds up to."""
+    N = T.numel()
+    dev = lp.device
+    alpha = torch.full((lp.shape[0],), float("nan"), dtype=torch.float32, device=dev)
+    beta = torch.full((lp.shape[0],), float("nan"), dtype=torch.float32, device=dev)
+    sa = torch.full((N,), float("nan"), dtype=torch.float32, device=dev)
+    sb = torch.full((N,), float("nan"), dtype=torch.float32, device=dev)
+    check(lib().ot_alpha_beta_guarded(ptr(lp), ptr(T), ptr(U), ptr(splits), ctypes.c_int32(N),
+                                      ctypes.c_int32(max_u1), ctypes.c_int32(int(one_sym_per_frame)),
+                                      ctypes.c_int64(rows), ptr(alpha), ptr(beta), ptr(sa), ptr(sb),
+                                      stream()))
+    return alpha, beta, sa, sb
+
+
 def gradient(logits, lp, den, alpha, beta, targets, T, U, splits, blank, from_log_softmax,
              one_sym_per_frame, grad_scale=1.0, grad=None, device_factor=None):
     """ot_gradient; with device_factor (a one-element device tensor) the two launches

@@ -255,3 +255,41 @@ def test_copy_floats(device):
     b = torch.zeros_like(a)
     cabi.copy_floats(a, b)
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("osf", [False, True])
+def test_guarded_lattice_launch(osf, device):
+    """ot_alpha_beta_guarded: the same results when the batch is what the caller believes, an
+    upper bound on the columns is fine, and nothing is written when the rows do not add up or a
+    length is out of range (the launch must be safe before the host has validated anything)."""
+    rng = np.random.default_rng(41)
+    T = np.array([9, 4, 17, 30], np.int32)
+    U = np.array([3, 0, 70, 12], np.int32)
+    if osf:
+        T = np.maximum(T, U + 2).astype(np.int32)
+    rows = int((T.astype(np.int64) * (U + 1)).sum())
+    lp = (-rng.random((rows, 2)) * 5 - 0.05).astype(np.float32)
+    dT, dU, dlp = _dev(T, device), _dev(U, device), _dev(lp, device)
+    splits, _ = cabi.row_splits(dT, dU, torch.zeros((4, 0), dtype=torch.int32, device=device))
+    want = cabi.alpha_beta(dlp, dT, dU, splits, int(U.max()) + 1, osf)
+    for max_u1 in (int(U.max()) + 1, 100):   # exact, and an upper bound in the same launch shape
+        got = cabi.alpha_beta_guarded(dlp, dT, dU, splits, max_u1, osf, rows)
+        for g, w in zip(got, want):
+            assert torch.equal(torch.nan_to_num(g, nan=7.0), torch.nan_to_num(w, nan=7.0))
+    # rows that do not add up: untouched outputs
+    for bad_rows in (rows - 1, rows + 5):
+        got = cabi.alpha_beta_guarded(dlp, dT, dU, splits, int(U.max()) + 1, osf, bad_rows)
+        assert all(torch.isnan(g).all() for g in got)
+    # a negative length that leaves the sum intact, and too few columns for one utterance: those
+    # workgroups write nothing, the others are unaffected by construction of the guard
+    T2, U2 = T.copy(), U.copy()
+    T2[1] = -T2[1]
+    dT2 = _dev(T2, device)
+    got = cabi.alpha_beta_guarded(dlp, dT2, dU, splits, int(U.max()) + 1, osf, rows)
+    a = got[0].cpu().numpy()
+    s0, s1 = int(splits[1].item()), int(splits[2].item())
+    assert np.isnan(a[s0:s1]).all()
+    got = cabi.alpha_beta_guarded(dlp, dT, dU, splits, 64, osf, rows)   # U = 70 needs 71 columns
+    a = got[0].cpu().numpy()
+    s2, s3 = int(splits[2].item()), int(splits[3].item())
+    assert np.isnan(a[s2:s3]).all() and not np.isnan(a[:s0]).any()
