@@ -9,21 +9,22 @@
 // the loss then starts from its gather step and the logits are read once, by the
 // gradient pass, instead of twice.
 //
-// Shape of the computation.  A workgroup of 8 waves owns 128 packed rows and walks
-// over the vocabulary in passes of 512 columns (one pass for V <= 512, so rows are
-// stored whole and the activations are read once); the waves form a 2 x 4 grid, a
-// wave holds a 128 x 64 block of logits^T in 8 accumulator tiles of 32 x 32
+// Shape of the computation.  A workgroup of 4 waves owns 128 packed rows and walks
+// over the vocabulary in passes of 256 columns; the waves form a 2 x 2 grid, a wave
+// holds a 128 x 64 block of logits^T in 8 accumulator tiles of 32 x 32
 // (v_mfma_f32_32x32x16).  The product is formed transposed (vocabulary along the
 // tile's rows, packed rows along its columns) because an accumulator lane then
 // holds 16 values of ONE packed row per tile: the running (max, sum) of the row
 // stays in that lane, with no cross-lane reduction until the very end, where the
-// lane's partner 32 lanes up and the 4 waves of the row are merged.  W and x
+// lane's partner 32 lanes up and the 2 waves of the row are merged.  W and x
 // stream through LDS in stages of 32 k-values (two buffers, 16-byte slots
 // XOR-swizzled against bank conflicts); the global loads of a stage are issued two
 // stages ahead into one of two register sets, because one stage of matrix work is
 // shorter than a trip to memory.  The bias initialises the accumulators.  The
 // stores go through a small wave-private LDS tile that turns the accumulator layout
-// into whole 128-byte pieces of rows.
+// into whole 128-byte pieces of rows.  Workgroups are persistent (two per compute
+// unit), so the loads of the next 128 rows are in flight while the last pass of the
+// current ones is stored.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -41,8 +42,8 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ unsigned as_u32(float v) { return __builtin_bit_cast(unsigned, v); }
 __device__ __forceinline__ float as_f32(unsigned v) { return __builtin_bit_cast(float, v); }
 
-constexpr int kProjRows = 128;     // packed rows per workgroup (2 waves)
-constexpr int kProjCols = 256;     // vocabulary columns per pass (2 waves)
+constexpr int kProjRows = 128;     // packed rows per workgroup (2 waves of 64)
+constexpr int kProjCols = 256;     // vocabulary columns per pass (2 waves of 128)
 constexpr int kProjK = 32;         // k-values per LDS stage
 constexpr int kProjThreads = 256;
 // ordinary (cached) stores: rows whose pitch is not a multiple of 128 bytes are written in
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
 
   // stage copy: a stage is 32 k-values = 4 chunks of 16 bytes per row; chunk cc of
   // row r lives in slot 4 r + (cc ^ ((r >> 2) & 3)).  Thread t moves pieces
-  // t, t + 512, ... of W (piece p: row p / 4, chunk p % 4) and piece t of x.
+  // t, t + 256, ... of W and of x (piece p: row p / 4, chunk p % 4).
   // Pieces t + 256 q of a thread are 64 rows apart: same chunk, same swizzle.
   const unsigned piece_src = ((unsigned)(tid >> 2) * (unsigned)D + 8u * (tid & 3)) * 2u;
   const unsigned piece_dst = (unsigned)(4 * (tid >> 2) + ((tid & 3) ^ ((tid >> 4) & 3))) * 16u;
