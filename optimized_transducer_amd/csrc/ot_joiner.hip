@@ -132,7 +132,11 @@ __global__ __launch_bounds__(kBlock) void joiner_pack_kernel(
 // The same with 2-byte output (float32 inputs and arithmetic, rounded to nearest
 // even): for a joiner whose projection runs in float16 / bfloat16, instead of a
 // float32 pack followed by a cast pass.  8 columns per thread, so that a thread
-// stores 16 bytes and a wave a contiguous 1 KiB.
+// stores 16 bytes and a wave a contiguous 1 KiB.  With tanh this kernel is bound
+// by its arithmetic, not its stores: 8 frames per workgroup (fastest of 2, 8, 16
+// at 4, 8 and 16 positions) spread the decoder loads and the index arithmetic
+// over four times as many outputs as the float32 kernel's 2.
+constexpr int kPackHalfFrames = 8;
 template <int ACT, class E>
 __global__ __launch_bounds__(kBlock) void joiner_pack_half_kernel(
     const float *__restrict__ enc, const float *__restrict__ dec,
@@ -141,7 +145,7 @@ __global__ __launch_bounds__(kBlock) void joiner_pack_half_kernel(
     unsigned short *__restrict__ out) {
   constexpr int VEC = 8;
   const int b = blockIdx.z;
-  const int t0 = blockIdx.y * kPackFrames;
+  const int t0 = blockIdx.y * kPackHalfFrames;
   const int T = min(logit_lengths[b], t_stride);
   if (t0 >= T) return;
   const int U1 = min(target_lengths[b] + 1, u_stride);
@@ -155,10 +159,10 @@ __global__ __launch_bounds__(kBlock) void joiner_pack_half_kernel(
   const int unit = slab * cpb + (threadIdx.x - phase * cpb);
   if (phase >= phases || unit >= nvec || u_begin >= U1) return;
   const int col = unit * VEC;
-  const int nt = min(kPackFrames, T - t0);
-  Vec<4> e[kPackFrames][2];
+  const int nt = min(kPackHalfFrames, T - t0);
+  Vec<4> e[kPackHalfFrames][2];
 #pragma unroll
-  for (int i = 0; i < kPackFrames; ++i)
+  for (int i = 0; i < kPackHalfFrames; ++i)
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
 #pragma unroll
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(kBlock) void joiner_pack_half_kernel(
       dn[1].load_cached(dp + (int64_t)(u + phases) * D + 4);
     }
 #pragma unroll
-    for (int i = 0; i < kPackFrames; ++i) {
+    for (int i = 0; i < kPackHalfFrames; ++i) {
       if (i < nt) {
         u32x4 y;
 #pragma unroll
@@ -442,12 +446,12 @@ int ot_joiner_pack_half(const float *enc, const float *dec, const int32_t *logit
       (out_dtype != OT_DTYPE_F16 && out_dtype != OT_DTYPE_BF16))
     return OT_E_BAD_ARG;
   if (!aligned16(enc) || !aligned16(dec) || !aligned16(out)) return OT_E_MISALIGNED;
-  if ((t_stride + kPackFrames - 1) / kPackFrames > 65535) return OT_E_TOO_LONG;
+  if ((t_stride + kPackHalfFrames - 1) / kPackHalfFrames > 65535) return OT_E_TOO_LONG;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int nvec = D / 8;
   const int cpb = nvec < kBlock ? nvec : kBlock;
   const dim3 grid((unsigned)(((nvec + cpb - 1) / cpb) * ((u_stride + kPackPositions - 1) / kPackPositions)),
-                  (unsigned)((t_stride + kPackFrames - 1) / kPackFrames), (unsigned)N);
+                  (unsigned)((t_stride + kPackHalfFrames - 1) / kPackHalfFrames), (unsigned)N);
   unsigned short *o = static_cast<unsigned short *>(out);
 #define OT_LAUNCH_PACKH(ACT_, E_)                                                              \
   hipLaunchKernelGGL((joiner_pack_half_kernel<ACT_, E_>), grid, dim3(kBlock), 0, s, enc, dec,  \
