@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # WRITE_SIZE runs scaled by the library's 1 GiB copy kernel (x2.000 / x1.000);
 # summary and commands in profiles/hbm_traffic_bench_asr_N32_V500.md.  Valid for
 # this workload and the kernel's current access pattern only.
-MEASURED_TRAFFIC_BYTES = {("asr_N32_V500", "grad_logits"): 3.0727e9}
+MEASURED_TRAFFIC_BYTES = {("asr_N32_V500", "grad_logits"): 3.1148e9}
 
 
 def make_workload(name):
@@ -348,6 +348,11 @@ def main():
         if args.loss_weight != 1.0:
             loss = loss * args.loss_weight
         loss.backward()
+        # what a training loop's zero_grad(set_to_none=True) does: with log-softmax
+        # input the gradient is a tensor of its own, and K of them kept alive would
+        # put K device allocations of (rows, V) floats into the timed region
+        # (with logits input the gradient is the buffer itself, and this frees nothing)
+        buf.grad = None
         return loss
 
     if args.calibrate_copy:

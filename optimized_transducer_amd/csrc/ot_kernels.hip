@@ -695,17 +695,24 @@ __global__ __launch_bounds__(kBlock) void row_coeff_kernel(
 // Flat pass over the (rows, V) array in units of VEC floats: unit i belongs to
 // row i / nvec.  Consecutive lanes touch consecutive 16-byte units, so every
 // wave instruction moves one aligned, contiguous 1 KiB whatever V is; a
-// workgroup owns kGradUnroll * 256 consecutive units and exists only for them
+// workgroup owns grad_unroll() * 256 consecutive units and exists only for them
 // (one-shot grid, non-temporal accesses: the measured optimum here both for the
 // read-modify-write stream of the logits input and for the write-only stream
 // of the log-softmax input).
-constexpr int kGradUnroll = 2;  // 2 x 16 bytes per thread: fastest of 1, 2, 4, 8 on MI355X
+#ifndef OT_GRAD_UNROLL_LOGITS
+#define OT_GRAD_UNROLL_LOGITS 1
+#endif
+// 16-byte units per thread, fastest of 1, 2, 4, 8 on MI355X for each stream: the
+// in-place stream of the logits input gains 2 % from 1 unit over 2, the write-only
+// stream of the log-softmax input loses 20 %.
+constexpr int grad_unroll(bool from_log_softmax) { return from_log_softmax ? 2 : OT_GRAD_UNROLL_LOGITS; }
 
 template <int VEC, bool FLS>
 __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
     const float *logits, float *grad, const float4 *__restrict__ coef_f,
     const int2 *__restrict__ coef_i, int64_t unit_begin, int64_t nunits, int nvec, float inv_nvec,
     double inv_nvec_d, float scale, const float *__restrict__ device_factor) {
+  constexpr int kGradUnroll = grad_unroll(FLS);
   // optional second factor that lives on the device (the upstream gradient of the loss)
   const float factor = device_factor ? *device_factor : 1.f;
   if (!FLS) scale *= factor;
@@ -1083,7 +1090,7 @@ static int launch_gradient_apply(const float *logits, const void *row_scratch, i
   const int vec = (aligned && V % 4 == 0) ? 4 : 1;
   const int nvec = V / vec;
   const int64_t unit_begin = row_begin * nvec, unit_end = row_end * nvec;
-  const int64_t per_block = (int64_t)kGradUnroll * kBlock;
+  const int64_t per_block = (int64_t)grad_unroll(from_log_softmax != 0) * kBlock;
   const int64_t blocks = (unit_end - unit_begin + per_block - 1) / per_block;
   if (blocks > INT32_MAX) return OT_E_BAD_ARG;
   const dim3 grid((unsigned)blocks);
