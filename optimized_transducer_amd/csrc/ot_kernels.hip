@@ -699,20 +699,20 @@ __global__ __launch_bounds__(kBlock) void row_coeff_kernel(
 // (one-shot grid, non-temporal accesses: the measured optimum here both for the
 // read-modify-write stream of the logits input and for the write-only stream
 // of the log-softmax input).
-#ifndef OT_GRAD_UNROLL_LOGITS
-#define OT_GRAD_UNROLL_LOGITS 1
-#endif
 // 16-byte units per thread, fastest of 1, 2, 4, 8 on MI355X for each stream: the
-// in-place stream of the logits input gains 2 % from 1 unit over 2, the write-only
-// stream of the log-softmax input loses 20 %.
-constexpr int grad_unroll(bool from_log_softmax) { return from_log_softmax ? 2 : OT_GRAD_UNROLL_LOGITS; }
+// in-place stream of the logits input gains 2-7 % from 1 unit over 2, the write-only
+// stream of the log-softmax input loses 20 %.  The 4-byte units of an unaligned
+// array or of a V that is no multiple of 4 keep 2 per thread.
+constexpr int grad_unroll(bool from_log_softmax, int vec) {
+  return (from_log_softmax || vec == 1) ? 2 : 1;
+}
 
 template <int VEC, bool FLS>
 __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
     const float *logits, float *grad, const float4 *__restrict__ coef_f,
     const int2 *__restrict__ coef_i, int64_t unit_begin, int64_t nunits, int nvec, float inv_nvec,
     double inv_nvec_d, float scale, const float *__restrict__ device_factor) {
-  constexpr int kGradUnroll = grad_unroll(FLS);
+  constexpr int kGradUnroll = grad_unroll(FLS, VEC);
   // optional second factor that lives on the device (the upstream gradient of the loss)
   const float factor = device_factor ? *device_factor : 1.f;
   if (!FLS) scale *= factor;
@@ -1090,7 +1090,7 @@ static int launch_gradient_apply(const float *logits, const void *row_scratch, i
   const int vec = (aligned && V % 4 == 0) ? 4 : 1;
   const int nvec = V / vec;
   const int64_t unit_begin = row_begin * nvec, unit_end = row_end * nvec;
-  const int64_t per_block = (int64_t)grad_unroll(from_log_softmax != 0) * kBlock;
+  const int64_t per_block = (int64_t)grad_unroll(from_log_softmax != 0, vec) * kBlock;
   const int64_t blocks = (unit_end - unit_begin + per_block - 1) / per_block;
   if (blocks > INT32_MAX) return OT_E_BAD_ARG;
   const dim3 grid((unsigned)blocks);
