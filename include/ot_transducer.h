@@ -218,6 +218,22 @@ int ot_scale_by_device_scalar(float *x, int64_t n, const float *factor,
 int ot_negative_sum(const float *scores, int32_t N, float scale, float *loss,
                     void *stream);
 
+/* ot_row_coefficients and ot_negative_sum in one launch: the per-row
+ * coefficients of the whole batch into `row_scratch`, and
+ * *loss = -loss_scale * sum_b scores[b] (transducer_loss.py:145-147) with the
+ * summation order, hence the bits, of ot_negative_sum.  `scores` are the
+ * per-utterance log-likelihoods ot_alpha_beta wrote on the same stream. */
+int ot_row_coefficients_loss(const float *lp, const float *den, const float *alpha,
+                             const float *beta, const int32_t *targets,
+                             const int32_t *logit_lengths,
+                             const int32_t *target_lengths,
+                             const int32_t *row_splits, int32_t N,
+                             int32_t targets_cols, int64_t rows, int32_t blank,
+                             int32_t from_log_softmax, int32_t one_sym_per_frame,
+                             float grad_scale, void *row_scratch,
+                             const float *scores, float loss_scale, float *loss,
+                             void *stream);
+
 /* Bytes of device scratch ot_transducer_loss needs for N utterances and
  * `rows` packed rows. */
 size_t ot_workspace_bytes(int32_t N, int64_t rows);

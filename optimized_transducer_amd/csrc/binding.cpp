@@ -151,11 +151,14 @@ inline int half_dtype(const torch::Tensor &t) {
 // With `coefficients` set, the (rows, V) gradient pass is left to
 // apply_deferred_gradient: the per-row coefficients go into a tensor of their own,
 // handed back through the pointer, and the returned gradient is None.
+// With `reduced_loss` set, the 0-dim loss -grad_scale * scores.sum() is computed as
+// well: by the row-coefficient launch where there is one, else by a launch of its own.
 std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
     torch::Tensor &logits, const torch::Tensor &targets, const torch::Tensor &logit_lengths,
     const torch::Tensor &target_lengths, int32_t blank, bool from_log_softmax,
     bool one_sym_per_frame, double grad_scale, torch::Tensor *coefficients,
-    const torch::optional<torch::Tensor> &denominators = torch::nullopt) {
+    const torch::optional<torch::Tensor> &denominators = torch::nullopt,
+    torch::Tensor *reduced_loss = nullptr) {
   const bool defer = coefficients != nullptr;
   const bool have_den = denominators.has_value() && denominators->defined();
   auto logits_arg = torch::TensorArg(logits, "logits", 0);
@@ -353,6 +356,12 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
     gradient = from_log_softmax ? torch::empty_like(logits) : logits;
   }
   void *p_grad = gradient.defined() ? gradient.data_ptr() : nullptr;
+  float *p_loss = nullptr;
+  bool loss_done = false;
+  if (reduced_loss) {
+    *reduced_loss = torch::empty({}, logits.options().dtype(torch::kFloat));
+    p_loss = reduced_loss->data_ptr<float>();
+  }
 
   // lattice + per-row coefficients of utterances [b0, b1) on stream `s`
   auto lattice_part = [&](int32_t b0, int32_t b1, hipStream_t s) {
@@ -362,7 +371,14 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
                                    one_sym_per_frame, b0, b1, alpha, beta,
                                    scores.data_ptr<float>(), scores_beta, s));
     }
-    if (want_grad) {
+    if (want_grad && p_loss && !loss_done && b0 == 0 && b1 == N) {
+      ScopedTimer timer("row_coeff", s);
+      OT_CHECK(ot_row_coefficients_loss(lp, den, alpha, beta, p_targets, p_T, p_U, row_splits,
+                                        (int32_t)N, (int32_t)S, rows, blank, from_log_softmax,
+                                        one_sym_per_frame, (float)grad_scale, coef,
+                                        scores.data_ptr<float>(), (float)grad_scale, p_loss, s));
+      loss_done = true;
+    } else if (want_grad) {
       ScopedTimer timer("row_coeff", s);
       OT_CHECK(ot_row_coefficients_range(lp, den, alpha, beta, p_targets, p_T, p_U, row_splits,
                                          (int32_t)N, (int32_t)S, rows, blank, from_log_softmax,
@@ -408,6 +424,11 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
     lattice_part(0, (int32_t)N, stream);
     gradient_part(0, (int32_t)N);
   }
+  if (p_loss && !loss_done) {
+    ScopedTimer timer("negative_sum", stream);
+    OT_CHECK(ot_negative_sum(scores.data_ptr<float>(), (int32_t)N, (float)grad_scale, p_loss,
+                             stream));
+  }
   if (gradient.defined()) return {scores, gradient};
   return {scores, torch::nullopt};
 }
@@ -444,6 +465,35 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_transducer_loss
                           one_sym_per_frame, grad_scale, &coefficients, denominators);
   if (coefficients.defined()) return {out.first, coefficients};
   return {out.first, torch::nullopt};
+}
+
+// compute_transducer_loss_scaled / _deferred that also return the reduced loss
+// -grad_scale * scores.sum() (transducer_loss.py:145-147 with grad_scale = 1 for
+// "sum" and 1/N for "mean"): (scores, gradient or coefficients or None, loss).
+std::tuple<torch::Tensor, torch::optional<torch::Tensor>, torch::Tensor>
+compute_transducer_loss_reduced(torch::Tensor &logits, const torch::Tensor &targets,
+                                const torch::Tensor &logit_lengths,
+                                const torch::Tensor &target_lengths, int32_t blank,
+                                bool from_log_softmax, bool one_sym_per_frame, double grad_scale,
+                                const torch::optional<torch::Tensor> &denominators) {
+  torch::Tensor loss;
+  auto out = compute_impl(logits, targets, logit_lengths, target_lengths, blank, from_log_softmax,
+                          one_sym_per_frame, grad_scale, nullptr, denominators, &loss);
+  return {out.first, out.second, loss};
+}
+
+std::tuple<torch::Tensor, torch::optional<torch::Tensor>, torch::Tensor>
+compute_transducer_loss_deferred_reduced(torch::Tensor &logits, const torch::Tensor &targets,
+                                         const torch::Tensor &logit_lengths,
+                                         const torch::Tensor &target_lengths, int32_t blank,
+                                         bool from_log_softmax, bool one_sym_per_frame,
+                                         double grad_scale,
+                                         const torch::optional<torch::Tensor> &denominators) {
+  torch::Tensor coefficients, loss;
+  auto out = compute_impl(logits, targets, logit_lengths, target_lengths, blank, from_log_softmax,
+                          one_sym_per_frame, grad_scale, &coefficients, denominators, &loss);
+  if (coefficients.defined()) return {out.first, coefficients, loss};
+  return {out.first, torch::nullopt, loss};
 }
 
 // Backward half: the one pass over (rows, V), with loss_grad (a one-element float
@@ -722,6 +772,18 @@ PYBIND11_MODULE(_optimized_transducer, m) {
         py::arg("denominators") = py::none(),
         "Everything but the (rows, V) gradient pass: returns (scores, per-row coefficients or "
         "None) and leaves logits untouched.");
+  m.def("compute_transducer_loss_reduced", &compute_transducer_loss_reduced, py::arg("logits"),
+        py::arg("targets"), py::arg("logit_lengths"), py::arg("target_lengths"), py::arg("blank"),
+        py::arg("from_log_softmax"), py::arg("one_sym_per_frame"), py::arg("grad_scale"),
+        py::arg("denominators") = py::none(),
+        "compute_transducer_loss_scaled that also returns the 0-dim loss "
+        "-grad_scale * scores.sum(): (scores, grad or None, loss).");
+  m.def("compute_transducer_loss_deferred_reduced", &compute_transducer_loss_deferred_reduced,
+        py::arg("logits"), py::arg("targets"), py::arg("logit_lengths"),
+        py::arg("target_lengths"), py::arg("blank"), py::arg("from_log_softmax"),
+        py::arg("one_sym_per_frame"), py::arg("grad_scale"), py::arg("denominators") = py::none(),
+        "compute_transducer_loss_deferred that also returns the 0-dim loss: "
+        "(scores, coefficients or None, loss).");
   m.def("apply_deferred_gradient", &apply_deferred_gradient, py::arg("logits"),
         py::arg("coefficients"), py::arg("from_log_softmax"), py::arg("grad_scale"),
         py::arg("loss_grad"),

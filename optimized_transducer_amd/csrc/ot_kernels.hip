@@ -636,6 +636,25 @@ __global__ __launch_bounds__(OT_MAX_U1) void alpha_beta_kernel(
 // column when a target equals blank.  col1 == kZeroRow marks an all-zero row
 // (outside the one-symbol-per-frame band, or likelihood not finite).
 
+// *loss = -scale * sum(scores) by one whole workgroup of kBlock threads, always in
+// the same order: thread i adds scores[i], scores[i + 256], ..., then the lanes of a
+// wave, then the four waves.
+__device__ __forceinline__ void negative_sum_block(const float *__restrict__ scores, int n,
+                                                   float scale, float *__restrict__ loss) {
+  __shared__ float s_part[kWavesPerBlock];
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < n; i += kBlock) acc += scores[i];
+  acc = group_allreduce<kWave>(acc, SumOp());
+  if ((threadIdx.x & (kWave - 1)) == 0) s_part[threadIdx.x / kWave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) t += s_part[w];
+    *loss = -(t * scale);
+  }
+}
+
 template <bool FLS>
 __global__ __launch_bounds__(kBlock) void row_coeff_kernel(
     const float *__restrict__ lp, const float *__restrict__ den,
@@ -643,8 +662,12 @@ __global__ __launch_bounds__(kBlock) void row_coeff_kernel(
     const int32_t *__restrict__ targets, const int32_t *__restrict__ logit_lengths,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits, int N,
     int targets_cols, int64_t row_begin, int64_t rows, int blank, int osf, float scale,
-    float4 *__restrict__ coef_f, int2 *__restrict__ coef_i) {
+    float4 *__restrict__ coef_f, int2 *__restrict__ coef_i, const float *__restrict__ scores,
+    float loss_scale, float *__restrict__ loss) {
   __shared__ BlockUtterances bu;
+  // optionally the reduced loss as well (the launch after the lattice kernel that
+  // would otherwise compute it takes longer to start than to run)
+  if (loss && blockIdx.x == 0) negative_sum_block(scores, N, loss_scale, loss);
   const int64_t row_first = row_begin + (int64_t)blockIdx.x * kBlock;
   const int64_t row_end = min(rows, row_first + kBlock);
   bu.load(row_splits, N, row_first, row_end - 1);
@@ -820,18 +843,7 @@ __global__ __launch_bounds__(kBlock) void scale_kernel(float *__restrict__ x, in
 __global__ __launch_bounds__(kBlock) void negative_sum_kernel(const float *__restrict__ scores,
                                                               int n, float scale,
                                                               float *__restrict__ loss) {
-  __shared__ float s_part[kWavesPerBlock];
-  float acc = 0.f;
-  for (int i = threadIdx.x; i < n; i += kBlock) acc += scores[i];
-  acc = group_allreduce<kWave>(acc, SumOp());
-  if ((threadIdx.x & (kWave - 1)) == 0) s_part[threadIdx.x / kWave] = acc;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float t = 0.f;
-#pragma unroll
-    for (int w = 0; w < kWavesPerBlock; ++w) t += s_part[w];
-    *loss = -(t * scale);
-  }
+  negative_sum_block(scores, n, scale, loss);
 }
 
 __global__ __launch_bounds__(kBlock) void copy_kernel(const float4 *__restrict__ src,
@@ -1031,20 +1043,21 @@ int ot_alpha_beta(const float *lp, const int32_t *logit_lengths, const int32_t *
                              stream);
 }
 
-int ot_row_coefficients_range(const float *lp, const float *den, const float *alpha,
-                              const float *beta, const int32_t *targets,
-                              const int32_t *logit_lengths, const int32_t *target_lengths,
-                              const int32_t *row_splits, int32_t N, int32_t targets_cols,
-                              int64_t rows, int32_t blank, int32_t from_log_softmax,
-                              int32_t one_sym_per_frame, float grad_scale, int64_t row_begin,
-                              int64_t row_end, void *row_scratch, void *stream) {
+static int launch_row_coefficients(const float *lp, const float *den, const float *alpha,
+                                   const float *beta, const int32_t *targets,
+                                   const int32_t *logit_lengths, const int32_t *target_lengths,
+                                   const int32_t *row_splits, int32_t N, int32_t targets_cols,
+                                   int64_t rows, int32_t blank, int32_t from_log_softmax,
+                                   int32_t one_sym_per_frame, float grad_scale, int64_t row_begin,
+                                   int64_t row_end, void *row_scratch, const float *scores,
+                                   float loss_scale, float *loss, void *stream) {
   if (!alpha || !beta || !logit_lengths || !target_lengths || !row_splits || !row_scratch ||
       N <= 0 || rows <= 0 || rows > INT32_MAX || blank < 0 || targets_cols < 0 ||
       (targets_cols > 0 && !targets) || (from_log_softmax ? !lp : !den) || row_begin < 0 ||
-      row_end > rows || row_begin > row_end)
+      row_end > rows || row_begin > row_end || (loss && !scores))
     return OT_E_BAD_ARG;
   if (reinterpret_cast<uintptr_t>(row_scratch) & 15) return OT_E_MISALIGNED;
-  if (row_begin == row_end) return 0;
+  if (row_begin == row_end) return loss ? ot_negative_sum(scores, N, loss_scale, loss, stream) : 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   float4 *coef_f = static_cast<float4 *>(row_scratch);
   int2 *coef_i = reinterpret_cast<int2 *>(coef_f + rows);
@@ -1052,12 +1065,41 @@ int ot_row_coefficients_range(const float *lp, const float *den, const float *al
   if (from_log_softmax)
     hipLaunchKernelGGL(row_coeff_kernel<true>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
                        targets, logit_lengths, target_lengths, row_splits, N, targets_cols,
-                       row_begin, row_end, blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
+                       row_begin, row_end, blank, one_sym_per_frame, grad_scale, coef_f, coef_i,
+                       scores, loss_scale, loss);
   else
     hipLaunchKernelGGL(row_coeff_kernel<false>, grid, dim3(kBlock), 0, s, lp, den, alpha, beta,
                        targets, logit_lengths, target_lengths, row_splits, N, targets_cols,
-                       row_begin, row_end, blank, one_sym_per_frame, grad_scale, coef_f, coef_i);
+                       row_begin, row_end, blank, one_sym_per_frame, grad_scale, coef_f, coef_i,
+                       scores, loss_scale, loss);
   return launch_status();
+}
+
+int ot_row_coefficients_range(const float *lp, const float *den, const float *alpha,
+                              const float *beta, const int32_t *targets,
+                              const int32_t *logit_lengths, const int32_t *target_lengths,
+                              const int32_t *row_splits, int32_t N, int32_t targets_cols,
+                              int64_t rows, int32_t blank, int32_t from_log_softmax,
+                              int32_t one_sym_per_frame, float grad_scale, int64_t row_begin,
+                              int64_t row_end, void *row_scratch, void *stream) {
+  return launch_row_coefficients(lp, den, alpha, beta, targets, logit_lengths, target_lengths,
+                                 row_splits, N, targets_cols, rows, blank, from_log_softmax,
+                                 one_sym_per_frame, grad_scale, row_begin, row_end, row_scratch,
+                                 nullptr, 0.f, nullptr, stream);
+}
+
+int ot_row_coefficients_loss(const float *lp, const float *den, const float *alpha,
+                             const float *beta, const int32_t *targets,
+                             const int32_t *logit_lengths, const int32_t *target_lengths,
+                             const int32_t *row_splits, int32_t N, int32_t targets_cols,
+                             int64_t rows, int32_t blank, int32_t from_log_softmax,
+                             int32_t one_sym_per_frame, float grad_scale, void *row_scratch,
+                             const float *scores, float loss_scale, float *loss, void *stream) {
+  if (!scores || !loss) return OT_E_BAD_ARG;
+  return launch_row_coefficients(lp, den, alpha, beta, targets, logit_lengths, target_lengths,
+                                 row_splits, N, targets_cols, rows, blank, from_log_softmax,
+                                 one_sym_per_frame, grad_scale, 0, rows, row_scratch, scores,
+                                 loss_scale, loss, stream);
 }
 
 int ot_row_coefficients(const float *lp, const float *den, const float *alpha, const float *beta,

@@ -62,7 +62,9 @@ class TransducerLossFunction(torch.autograd.Function):
 
         ctx.deferred = None
         if defer_gradient:
-            scores, coefficients = _optimized_transducer.compute_transducer_loss_deferred(
+            # loss = -1 * scores, then .mean() or .sum() (reference transducer_loss.py:145-147),
+            # computed by the launch that makes the per-row coefficients
+            _, coefficients, loss = _optimized_transducer.compute_transducer_loss_deferred_reduced(
                 logits=logits,
                 targets=targets,
                 logit_lengths=logit_lengths,
@@ -78,9 +80,12 @@ class TransducerLossFunction(torch.autograd.Function):
                 # backward is then reported instead of giving a wrong gradient
                 ctx.save_for_backward(logits)
                 ctx.deferred = (coefficients, from_log_softmax, grad_scale)
-            return _optimized_transducer.negative_sum(scores, grad_scale)
+            return loss
 
-        scores, grad = _optimized_transducer.compute_transducer_loss_scaled(
+        # loss = -1 * scores, then .mean() or .sum() (reference transducer_loss.py:145-147):
+        # part of the launch that makes the per-row coefficients when there is a gradient,
+        # a launch of its own otherwise
+        _, grad, loss = _optimized_transducer.compute_transducer_loss_reduced(
             logits=logits,
             targets=targets,
             logit_lengths=logit_lengths,
@@ -91,9 +96,6 @@ class TransducerLossFunction(torch.autograd.Function):
             grad_scale=grad_scale,
             denominators=denominators,
         )
-
-        # loss = -1 * scores, then .mean() or .sum() (reference transducer_loss.py:145-147)
-        loss = _optimized_transducer.negative_sum(scores, grad_scale)
 
         ctx.grad = grad
         return loss

@@ -204,6 +204,27 @@ def joiner_unpack_grad(grad_out, enc, dec, T, U, splits, activation):
     return ge, gd
 
 
+def row_coefficients(lp, den, alpha, beta, targets, T, U, splits, blank, from_log_softmax,
+                     one_sym_per_frame, grad_scale=1.0, scores=None, loss_scale=1.0):
+    """ot_row_coefficients, or ot_row_coefficients_loss when `scores` is given.
+    Returns (row scratch as bytes, loss or None)."""
+    rows = alpha.numel()
+    cols = targets.shape[1]
+    scratch = torch.zeros(lib().ot_gradient_scratch_bytes(ctypes.c_int64(rows)), dtype=torch.uint8,
+                          device=alpha.device)
+    head = (ptr(lp), ptr(den), ptr(alpha), ptr(beta), ptr(targets if cols else None), ptr(T), ptr(U),
+            ptr(splits), ctypes.c_int32(T.numel()), ctypes.c_int32(cols), ctypes.c_int64(rows),
+            ctypes.c_int32(blank), ctypes.c_int32(int(from_log_softmax)),
+            ctypes.c_int32(int(one_sym_per_frame)), ctypes.c_float(grad_scale), ptr(scratch))
+    if scores is None:
+        check(lib().ot_row_coefficients(*head, stream()))
+        return scratch, None
+    loss = torch.full((1,), float("nan"), dtype=torch.float32, device=alpha.device)
+    check(lib().ot_row_coefficients_loss(*head, ptr(scores), ctypes.c_float(loss_scale), ptr(loss),
+                                         stream()))
+    return scratch, loss
+
+
 def negative_sum(scores, scale):
     loss = torch.full((1,), float("nan"), dtype=torch.float32, device=scores.device)
     check(lib().ot_negative_sum(ptr(scores), ctypes.c_int32(scores.numel()), ctypes.c_float(scale),

@@ -6,6 +6,8 @@ asserted per stage without the fp32 cancellation noise that an end-to-end
 comparison of two fp32 implementations carries (that comparison lives in
 test_gpu_end_to_end.py).
 """
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -248,6 +250,43 @@ def test_negative_sum(device):
             assert cabi.negative_sum(d, scale).item() == got
     inf = _dev(np.array([-1.0, -np.inf], np.float32), device)
     assert cabi.negative_sum(inf, 1.0).item() == np.inf
+
+
+@pytest.mark.parametrize("fls", [False, True])
+def test_row_coefficients_with_the_loss_in_the_same_launch(fls, device):
+    # ot_row_coefficients_loss = ot_row_coefficients + ot_negative_sum: the same coefficient
+    # bytes and the same bits of the loss (transducer_loss.py:145-147), twice in a row
+    _, T, U, tg, x, blank, osf = CASES[0]
+    xin = helpers.log_softmax32(x) if fls else x
+    _, _, parts = helpers.oracle_full(xin, tg, T, U, blank, fls, osf)
+    ninf = lambda v: np.where(np.isnan(v), -np.inf, v).astype(np.float32)  # noqa: E731
+    dT, dU, dtg = _dev(T, device), _dev(U, device), _dev(tg, device)
+    splits, _ = cabi.row_splits(dT, dU, dtg)
+    den = None if fls else _dev(parts["den"], device)
+    args = (_dev(ninf(parts["lp"]), device), den, _dev(ninf(parts["alpha"]), device),
+            _dev(ninf(parts["beta"]), device), dtg, dT, dU, splits, blank, fls, osf)
+    rng = np.random.default_rng(11)
+    for n_scale in (1.0, 1.0 / len(T)):
+        scores = _dev((-rng.random(len(T)) * 300).astype(np.float32), device)
+        plain, none = cabi.row_coefficients(*args, grad_scale=n_scale)
+        assert none is None
+        want = cabi.negative_sum(scores, n_scale)
+        for _ in range(2):
+            fused, loss = cabi.row_coefficients(*args, grad_scale=n_scale, scores=scores,
+                                                loss_scale=n_scale)
+            assert torch.equal(fused, plain)
+            assert torch.equal(loss, want), (loss.item(), want.item())
+    # a missing scores or loss pointer is refused before anything is launched
+    rows = int(parts["alpha"].size)
+    scratch = torch.zeros(cabi.lib().ot_gradient_scratch_bytes(ctypes.c_int64(rows)),
+                          dtype=torch.uint8, device=device)
+    rc = cabi.lib().ot_row_coefficients_loss(
+        cabi.ptr(args[0]), cabi.ptr(den), cabi.ptr(args[2]), cabi.ptr(args[3]), cabi.ptr(dtg),
+        cabi.ptr(dT), cabi.ptr(dU), cabi.ptr(splits), ctypes.c_int32(len(T)),
+        ctypes.c_int32(tg.shape[1]), ctypes.c_int64(rows), ctypes.c_int32(blank),
+        ctypes.c_int32(int(fls)), ctypes.c_int32(int(osf)), ctypes.c_float(1.0), cabi.ptr(scratch),
+        None, ctypes.c_float(1.0), None, cabi.stream())
+    assert rc != 0
 
 
 def test_copy_floats(device):
