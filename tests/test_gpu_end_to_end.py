@@ -76,6 +76,27 @@ def test_python_api_matches_oracle(fls, osf, reduction, device):
     assert np.abs(got - g64).max() <= 2 * np.abs(want_grad - g64).max() + 1e-6
 
 
+@pytest.mark.parametrize("reduction", ["mean", "sum"])
+@pytest.mark.parametrize("defer", [False, True])
+def test_loss_has_the_same_bits_with_and_without_a_gradient(defer, reduction, device):
+    # with a gradient the loss is reduced inside the row-coefficient launch, without one by
+    # a launch of its own (transducer_loss.py:145-147 either way): same summation, same bits,
+    # and equal to the reduction of the binding's per-utterance scores
+    import optimized_transducer_amd as ot
+    from optimized_transducer_amd import _optimized_transducer as ext
+    w = workloads.asr_batch(N=7, V=33, scale=0.1)
+    x = torch.from_numpy(w.logits_numpy()).to(device)
+    tg, T, U = (torch.from_numpy(a).to(device) for a in (w.targets, w.logit_lengths, w.target_lengths))
+    plain = ot.transducer_loss(x.clone(), tg, T, U, w.blank, False, False, reduction)
+    with_grad = ot.transducer_loss(x.clone().requires_grad_(True), tg, T, U, w.blank, False, False,
+                                   reduction, defer_gradient=defer)
+    scores, _ = ext.compute_transducer_loss(logits=x.clone(), targets=tg, logit_lengths=T,
+                                            target_lengths=U, blank=w.blank, from_log_softmax=False,
+                                            one_sym_per_frame=False)
+    want = ext.negative_sum(scores, 1.0 / w.N if reduction == "mean" else 1.0)
+    assert torch.equal(plain, want) and torch.equal(with_grad.detach(), want)
+
+
 def test_in_place_and_aliasing_semantics(device):
     import optimized_transducer_amd as ot
     w = workloads.tiny()
