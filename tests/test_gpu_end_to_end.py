@@ -97,6 +97,40 @@ def test_loss_has_the_same_bits_with_and_without_a_gradient(defer, reduction, de
     assert torch.equal(plain, want) and torch.equal(with_grad.detach(), want)
 
 
+@pytest.mark.parametrize("big", [False, True], ids=["small", "large"])
+def test_random_batches_against_the_oracle(big, device):
+    # every option drawn at random per batch: recursion, input kind, reduction, blank anywhere in
+    # [0, V), V with and without a factor of 4, an upstream gradient, the deferred mode
+    import optimized_transducer_amd as ot
+    rng = np.random.default_rng(20261125 + big)
+    for case in range(12 if big else 60):
+        osf, fls, defer = (bool(rng.integers(0, 2)) for _ in range(3))
+        N = int(rng.integers(1, 5 if big else 7))
+        V = int(rng.integers(2, 700 if big else 70))
+        tmax = int(rng.integers(1, 300 if big else 60))
+        umax = int(rng.integers(0, 160 if big else 20))
+        T, U, tg, x = helpers.random_batch(rng, N, tmax, umax, V, one_sym_per_frame=osf)
+        blank = int(rng.integers(0, V))
+        reduction = ("mean", "sum")[int(rng.integers(0, 2))]
+        up = float(rng.choice([1.0, 3.0, 0.5]))
+        xin = helpers.log_softmax32(x) if fls else x
+        want_loss, want_grad = oracle.transducer_loss(xin.copy(), tg, T, U, blank, fls, osf,
+                                                      reduction, loss_grad=up)
+        s, _ = oracle.compute_transducer_loss(xin.copy(), tg, T, U, blank, fls, osf)
+        logits = _dev(xin.copy(), device).requires_grad_(True)
+        loss = ot.transducer_loss(logits, _dev(tg, device), _dev(T, device), _dev(U, device), blank,
+                                  fls, one_sym_per_frame=osf, reduction=reduction,
+                                  defer_gradient=defer)
+        (loss * up if up != 1.0 else loss).backward()
+        what = dict(case=case, osf=osf, fls=fls, defer=defer, T=T.tolist(), U=U.tolist(), V=V,
+                    blank=blank, reduction=reduction, up=up)
+        assert np.allclose(loss.item(), want_loss, rtol=RTOL, atol=ATOL), what
+        scale = up / (N if reduction == "mean" else 1)
+        tol = scale * helpers.lattice_noise_tolerance(want_grad / scale, helpers.per_row(s, T, U))
+        err = np.abs(logits.grad.cpu().numpy() - want_grad)
+        assert (err <= tol).all(), (what, err.max())
+
+
 def test_in_place_and_aliasing_semantics(device):
     import optimized_transducer_amd as ot
     w = workloads.tiny()
