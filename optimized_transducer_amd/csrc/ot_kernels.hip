@@ -718,29 +718,35 @@ __global__ __launch_bounds__(kBlock) void row_coeff_kernel(
 // Flat pass over the (rows, V) array in units of VEC floats: unit i belongs to
 // row i / nvec.  Consecutive lanes touch consecutive 16-byte units, so every
 // wave instruction moves one aligned, contiguous 1 KiB whatever V is; a
-// workgroup owns grad_unroll() * 256 consecutive units and exists only for them
+// workgroup owns grad_unroll() * grad_block() consecutive units and exists only for them
 // (one-shot grid, non-temporal accesses: the measured optimum here both for the
 // read-modify-write stream of the logits input and for the write-only stream
 // of the log-softmax input).
-// 16-byte units per thread, fastest of 1, 2, 4, 8 on MI355X for each stream: the
-// in-place stream of the logits input gains 2-7 % from 1 unit over 2, the write-only
-// stream of the log-softmax input loses 20 %.  The 4-byte units of an unaligned
-// array or of a V that is no multiple of 4 keep 2 per thread.
+// Threads per workgroup and 16-byte units per thread, measured per stream on MI355X.
+// In-place stream of the logits input: 256 x 1 (2-7 % faster than 256 x 2; 64 x 1 the
+// same, 128 x 1, 128 x 2, 64 x 2 and 64 x 4 slower).  Write-only stream of the
+// log-softmax input: 64 x 2, one wave per workgroup (6 % faster than 256 x 2, 3 % than
+// 128 x 2; 64 x 4, 128 x 4 slower, 128 x 1 and 256 x 1 20 % slower).  The 4-byte units of
+// an unaligned array or of a V that is no multiple of 4 keep 256 x 2.
 constexpr int grad_unroll(bool from_log_softmax, int vec) {
   return (from_log_softmax || vec == 1) ? 2 : 1;
 }
+constexpr int grad_block(bool from_log_softmax, int vec) {
+  return (from_log_softmax && vec == 4) ? kWave : kBlock;
+}
 
 template <int VEC, bool FLS>
-__global__ __launch_bounds__(kBlock) void grad_flat_kernel(
+__global__ __launch_bounds__(grad_block(FLS, VEC)) void grad_flat_kernel(
     const float *logits, float *grad, const float4 *__restrict__ coef_f,
     const int2 *__restrict__ coef_i, int64_t unit_begin, int64_t nunits, int nvec, float inv_nvec,
     double inv_nvec_d, float scale, const float *__restrict__ device_factor) {
   constexpr int kGradUnroll = grad_unroll(FLS, VEC);
+  constexpr int kGradBlock = grad_block(FLS, VEC);
   // optional second factor that lives on the device (the upstream gradient of the loss)
   const float factor = device_factor ? *device_factor : 1.f;
   if (!FLS) scale *= factor;
   // this launch covers units [unit_begin, nunits)
-  const int64_t base = unit_begin + (int64_t)blockIdx.x * (kGradUnroll * kBlock);
+  const int64_t base = unit_begin + (int64_t)blockIdx.x * (kGradUnroll * kGradBlock);
   // base / nvec through a double reciprocal (exact below 2^53) and one correction step
   int64_t row_base = (int64_t)((double)base * inv_nvec_d);
   {
@@ -750,7 +756,7 @@ __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
   const int rem_base = (int)(base - row_base * nvec);
   // the workgroup's units as raw buffers: the tail of the last workgroup needs no branch
   const unsigned span_bytes =
-      (unsigned)min((int64_t)(kGradUnroll * kBlock), nunits - base) * (VEC * 4u);
+      (unsigned)min((int64_t)(kGradUnroll * kGradBlock), nunits - base) * (VEC * 4u);
   const __amdgpu_buffer_rsrc_t in_buf = make_buffer(FLS ? grad : logits + base * VEC, span_bytes);
   const __amdgpu_buffer_rsrc_t out_buf = make_buffer(grad + base * VEC, span_bytes);
 
@@ -758,7 +764,7 @@ __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
   int rows[kGradUnroll], col0[kGradUnroll];
 #pragma unroll
   for (int k = 0; k < kGradUnroll; ++k) {
-    const int local = k * kBlock + (int)threadIdx.x;
+    const int local = k * kGradBlock + (int)threadIdx.x;
     if (!FLS) x[k].load_buffer(in_buf, (unsigned)local * (VEC * 4u));
     // idx < nvec + kGradUnroll*256 is exact in float; one correction step fixes the quotient
     const int idx = rem_base + local;
@@ -770,7 +776,7 @@ __global__ __launch_bounds__(kBlock) void grad_flat_kernel(
   const int64_t last_row = (nunits - 1) / nvec;
 #pragma unroll
   for (int k = 0; k < kGradUnroll; ++k) {
-    const int local = k * kBlock + (int)threadIdx.x;
+    const int local = k * kGradBlock + (int)threadIdx.x;
     const int64_t row = min(row_base + rows[k], last_row);
     const float4 f = coef_f[row];
     const int2 ci = coef_i[row];
@@ -1132,13 +1138,14 @@ static int launch_gradient_apply(const float *logits, const void *row_scratch, i
   const int vec = (aligned && V % 4 == 0) ? 4 : 1;
   const int nvec = V / vec;
   const int64_t unit_begin = row_begin * nvec, unit_end = row_end * nvec;
-  const int64_t per_block = (int64_t)grad_unroll(from_log_softmax != 0, vec) * kBlock;
+  const int gblock = grad_block(from_log_softmax != 0, vec);
+  const int64_t per_block = (int64_t)grad_unroll(from_log_softmax != 0, vec) * gblock;
   const int64_t blocks = (unit_end - unit_begin + per_block - 1) / per_block;
   if (blocks > INT32_MAX) return OT_E_BAD_ARG;
   const dim3 grid((unsigned)blocks);
   const float inv_nvec = 1.0f / (float)nvec;
 #define OT_LAUNCH_GRAD(VEC_, FLS_)                                                            \
-  hipLaunchKernelGGL((grad_flat_kernel<VEC_, FLS_>), grid, dim3(kBlock), 0, s, logits, grad,  \
+  hipLaunchKernelGGL((grad_flat_kernel<VEC_, FLS_>), grid, dim3(gblock), 0, s, logits, grad,  \
                      coef_f, coef_i, unit_begin, unit_end, nvec, inv_nvec, 1.0 / (double)nvec,       \
                      grad_scale, device_factor)
   if (from_log_softmax) {
