@@ -31,6 +31,7 @@ extern "C" {
 #define OT_E_BAD_ARG (-1)       /* null pointer / non-positive size            */
 #define OT_E_TOO_LONG (-2)      /* max(U)+1 exceeds OT_MAX_U1                  */
 #define OT_E_MISALIGNED (-3)    /* logits / grad not 4-byte aligned            */
+#define OT_E_TOO_LARGE (-4)     /* batch exceeds OT_STATIC_WORKSPACE_BYTES     */
 
 /* Largest U+1 the lattice kernels handle (one thread per u, one workgroup per
  * utterance and direction).  The reference's CUDA path has the same bound
@@ -255,6 +256,30 @@ int ot_transducer_loss(const float *logits, const int32_t *targets,
                        float grad_scale, void *workspace,
                        size_t workspace_bytes, float *scores, float *grad,
                        ot_batch_status *status, void *stream);
+
+/* ot_transducer_loss for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It
+ * has no counterpart in the reference, whose launchers allocate every temporary
+ * with torch::empty (cuda.cu:416-446).  Same arguments, kernels and results as
+ * ot_transducer_loss without `workspace`: the temporaries live in an array of
+ * OT_STATIC_WORKSPACE_BYTES that is part of the library's device image (every GPU
+ * the library runs on holds its own copy until the process ends).  The call
+ * itself calls no hipMalloc / hipFree.  A batch with
+ * ot_workspace_bytes(N, rows) > OT_STATIC_WORKSPACE_BYTES (about 44 bytes per
+ * packed row: 1.1 million rows) returns OT_E_TOO_LARGE and launches nothing.
+ * All calls on one GPU share the array: calls that overlap in time on one GPU
+ * (two streams, two threads) race; calls on one stream are ordered and need no
+ * clearing in between.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress); make it outside any graph capture. */
+#define OT_STATIC_WORKSPACE_BYTES (48u << 20)
+int ot_transducer_loss_static(const float *logits, const int32_t *targets,
+                              const int32_t *logit_lengths,
+                              const int32_t *target_lengths, int32_t N,
+                              int32_t targets_cols, int64_t rows, int32_t V,
+                              int32_t blank, int32_t from_log_softmax,
+                              int32_t one_sym_per_frame, int32_t max_u1,
+                              float grad_scale, float *scores, float *grad,
+                              ot_batch_status *status, void *stream);
 
 /* ---- packed joiner input: the data format on the input side of the loss ----
  *

@@ -20,6 +20,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "ot_device.hip.h"
@@ -1255,6 +1256,59 @@ int ot_transducer_loss(const float *logits, const int32_t *targets, const int32_
   return rc;
 }
 
+// ---------------------------------------------------------------------------
+// The whole path for callers that cannot allocate: the workspace is a file-scope
+// device array.  Its name is a host-side stand-in, not a device address: the
+// address on each device is looked up once with hipGetSymbolAddress and only that
+// pointer is ever handed to a kernel.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[OT_STATIC_WORKSPACE_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];  // address of `scratch` on each device, once known
+
+// Address of this device's copy of `scratch` (every GPU holds its own).
+int static_scratch(void **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return OT_E_BAD_ARG;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return OT_E_BAD_ARG;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+}  // namespace
+
+int ot_transducer_loss_static(const float *logits, const int32_t *targets,
+                              const int32_t *logit_lengths, const int32_t *target_lengths,
+                              int32_t N, int32_t targets_cols, int64_t rows, int32_t V,
+                              int32_t blank, int32_t from_log_softmax, int32_t one_sym_per_frame,
+                              int32_t max_u1, float grad_scale, float *scores, float *grad,
+                              ot_batch_status *status, void *stream) {
+  if (N <= 0 || rows <= 0) return OT_E_BAD_ARG;
+  // sizes first: a batch that does not fit is refused before anything touches the device
+  if (rows > INT32_MAX || ot_workspace_bytes(N, rows) > (size_t)OT_STATIC_WORKSPACE_BYTES)
+    return OT_E_TOO_LARGE;
+  void *ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc) return rc;
+  // every slice of the workspace is written in full before it is read (row offsets,
+  // denominators, log-probabilities, every lattice cell, every row's coefficients), so
+  // what the previous call left in the array needs no clearing
+  return ot_transducer_loss(logits, targets, logit_lengths, target_lengths, N, targets_cols, rows,
+                            V, blank, from_log_softmax, one_sym_per_frame, max_u1, grad_scale, ws,
+                            (size_t)OT_STATIC_WORKSPACE_BYTES, scores, grad, status, stream);
+}
+
 int ot_negative_sum(const float *scores, int32_t N, float scale, float *loss, void *stream) {
   if (!scores || !loss || N <= 0) return OT_E_BAD_ARG;
   hipLaunchKernelGGL(negative_sum_kernel, dim3(1), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
@@ -1280,6 +1334,9 @@ const char *ot_error_string(int code) {
     case OT_E_BAD_ARG: return "ot: null pointer, non-positive size or out-of-range argument";
     case OT_E_TOO_LONG: return "ot: max(target_lengths)+1 exceeds OT_MAX_U1";
     case OT_E_MISALIGNED: return "ot: float buffer is not 4-byte aligned";
+    case OT_E_TOO_LARGE:
+      return "ot: the batch needs more workspace than OT_STATIC_WORKSPACE_BYTES; use "
+             "ot_transducer_loss with a workspace of ot_workspace_bytes(N, rows)";
     default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "ot: unknown error";
   }
 }
