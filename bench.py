@@ -22,11 +22,24 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs scaled by the library's 1 GiB copy kernel (x2.000 / x1.000);
-# summary and commands in profiles/hbm_traffic_bench_asr_N32_V500.md.  Valid for
-# this workload and the kernel's current access pattern only.
-MEASURED_TRAFFIC_BYTES = {("asr_N32_V500", "grad_logits"): 3.1148e9}
+
+
+def measured_traffic(workload_name, kernel):
+    """HBM bytes per launch of `kernel` on `workload_name` as a committed counter
+    summary records them (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
+    counters on the library's 1 GiB copy kernel): the line
+    `traffic_bytes_per_launch <workload> <kernel> <bytes> source_sha <sha>` of a
+    profiles/hbm_traffic_*.md file.  Returns (bytes, source) or (None, None): nothing
+    is echoed that is not on file, and the source names the commit it was measured at."""
+    import glob
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "hbm_traffic_*.md"))):
+        with open(path) as f:
+            for line in f:
+                parts = line.replace("`", " ").split()
+                if (len(parts) >= 6 and parts[0] == "traffic_bytes_per_launch"
+                        and parts[1] == workload_name and parts[2] == kernel):
+                    return float(parts[3]), "profiles/%s @ %s" % (os.path.basename(path), parts[5])
+    return None, None
 
 
 def make_workload(name):
@@ -55,9 +68,22 @@ def algorithmic_bytes(w, esize=4):
             "grad_logits": (2 * esize * V + 20) * R}
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(w, logits_host, max_seconds=30.0):
     """The reference's CPU path (oracle/_ref) or, failing that, the C port, on
-    the same batch; bounded to about max_seconds of CPU time."""
+    the same batch; bounded to about max_seconds of CPU time.  Returns the record
+    for the JSON line and the (scores, loss, gradient) of the last run, which the
+    parity check compares the GPU's results with."""
     import numpy as np
     import torch
     from oracle import oracle, ref_loader
@@ -67,6 +93,8 @@ def cpu_baseline(w, logits_host, max_seconds=30.0):
     tg = torch.from_numpy(w.targets)
     T = torch.from_numpy(w.logit_lengths)
     U = torch.from_numpy(w.target_lengths)
+
+    result = {}
 
     def once():
         x = logits_host.clone()
@@ -82,10 +110,19 @@ def cpu_baseline(w, logits_host, max_seconds=30.0):
                 if w.reduction == "mean":
                     grad /= w.N
                 grad.mul_(torch.ones(()))  # backward's mul_(loss_grad)
+            dt = time.perf_counter() - t0
+            result.update(scores=scores.detach(), loss=float(loss), grad=grad.detach())
         else:
-            oracle.transducer_loss(x.numpy(), w.targets, w.logit_lengths, w.target_lengths,
-                                   w.blank, w.from_log_softmax, w.one_sym_per_frame, w.reduction)
-        return time.perf_counter() - t0
+            loss, grad = oracle.transducer_loss(x.numpy(), w.targets, w.logit_lengths,
+                                                w.target_lengths, w.blank, w.from_log_softmax,
+                                                w.one_sym_per_frame, w.reduction)
+            dt = time.perf_counter() - t0
+            scores, _ = oracle.compute_transducer_loss(
+                logits_host.numpy().copy(), w.targets, w.logit_lengths, w.target_lengths, w.blank,
+                w.from_log_softmax, w.one_sym_per_frame, want_grad=False)
+            result.update(scores=torch.from_numpy(scores), loss=float(loss),
+                          grad=torch.from_numpy(grad))
+        return dt
 
     times = [once()]
     while len(times) < 3 and sum(times) + times[-1] < max_seconds:
@@ -94,6 +131,7 @@ def cpu_baseline(w, logits_host, max_seconds=30.0):
     kind = "reference" if ref is not None else "port"
     return {
         "value": w.N / best, "unit": "utterances/s", "cores": threads if ref is not None else 1,
+        "os_cpu_count": os.cpu_count(), "cpu_model": cpu_model(),
         "kind": kind,
         "sample": "%d full batch(es) of workload %s (N=%d, rows=%d, V=%d), median of %d; "
                   "%s" % (len(times), w.name, w.N, w.rows, w.V, len(times),
@@ -101,7 +139,78 @@ def cpu_baseline(w, logits_host, max_seconds=30.0):
                           "as the reference runs them" % threads if ref is not None
                           else "single-threaded C port of the reference's CPU path"),
         "seconds_per_batch": best,
+    }, result
+
+
+def parity_record(w, args, pristine, targets, T, U, ref, with_f64):
+    """The timed workload once more through the shipped Python entry point, outside
+    the timed region, against what the CPU baseline computed for the same batch
+    (the compiled reference, float32): the parity gate of this run."""
+    import numpy as np
+    import torch
+    import optimized_transducer_amd as ot
+    from optimized_transducer_amd import _optimized_transducer as ext
+    from oracle import oracle
+
+    buf = pristine.clone().requires_grad_(True)
+    loss = ot.transducer_loss(buf, targets, T, U, w.blank, w.from_log_softmax, w.one_sym_per_frame,
+                              w.reduction, defer_gradient=args.defer_gradient)
+    (loss * args.loss_weight if args.loss_weight != 1.0 else loss).backward()
+    got_grad = buf.grad.float().cpu()
+    got_loss = float(loss)
+    scores, _ = ext.compute_transducer_loss(
+        logits=pristine.clone(), targets=targets, logit_lengths=T, target_lengths=U, blank=w.blank,
+        from_log_softmax=w.from_log_softmax, one_sym_per_frame=w.one_sym_per_frame)
+    got_scores = scores.cpu()
+    del buf, scores
+
+    ref_grad = ref["grad"] if args.loss_weight == 1.0 else ref["grad"] * args.loss_weight
+    diff = (got_grad - ref_grad).abs_()
+    big = ref_grad.abs() > 1e-4
+    within = diff <= 1e-5 + 1e-5 * ref_grad.abs()
+    rec = {
+        "entry_point": "optimized_transducer_amd.transducer_loss(...).backward()",
+        "against": "the CPU baseline's output for the same batch (float32)",
+        "loss": got_loss, "loss_reference": ref["loss"],
+        "loss_rel_err": abs(got_loss - ref["loss"]) / max(abs(ref["loss"]), 1e-30),
+        "scores_max_rel_err": float(((got_scores - ref["scores"]).abs()
+                                     / ref["scores"].abs().clamp_min(1e-30)).max()),
+        "grad_max_abs_err": float(diff.max()),
+        "grad_max_rel_err_over_1e-4": float((diff[big] / ref_grad[big].abs()).max()) if bool(big.any()) else 0.0,
+        "grad_entries_over_1e-4": int(big.sum()),
+        "grad_frac_within_1e-5": float(within.double().mean()),
+        "grad_allclose_rtol1e-5_atol1e-5": bool(within.all()),
+        "scores_allclose_rtol1e-5_atol1e-5": bool(torch.allclose(got_scores, ref["scores"], rtol=1e-5, atol=1e-5)),
     }
+    del diff, big, within
+    if with_f64:
+        # the same recursions in float64 as the arbiter between two float32 evaluations
+        x = pristine.float().cpu().numpy()
+        s64, g64, m64 = oracle.compute_transducer_loss(
+            x, w.targets, w.logit_lengths, w.target_lengths, w.blank, w.from_log_softmax,
+            w.one_sym_per_frame, dtype=np.float64, return_magnitude=True)
+        del x
+        scale = args.loss_weight / (w.N if w.reduction == "mean" else 1.0)
+        g64 *= scale
+        m64 *= scale
+        sizes = w.logit_lengths.astype(np.int64) * (w.target_lengths.astype(np.int64) + 1)
+        unit = np.finfo(np.float32).eps * np.repeat(np.abs(s64), sizes)[:, None] * m64
+        ok = unit > 1e-30
+        rec["float64"] = {}
+        dgr = np.abs(got_grad.numpy() - ref_grad.numpy())
+        rec["grad_max_err_in_noise_units"] = float((dgr[ok] / unit[ok]).max())
+        del dgr
+        for name, g, sc in (("gpu", got_grad.numpy(), got_scores.numpy()),
+                            ("reference", ref_grad.numpy(), ref["scores"].numpy())):
+            d = np.abs(g - g64)
+            rec["float64"][name] = {
+                "grad_max_abs_err": float(d.max()),
+                # in units of eps * |log-likelihood| * (sum of the entry's exponentials)
+                "grad_max_err_in_noise_units": float((d[ok] / unit[ok]).max()),
+                "scores_max_rel_err": float((np.abs(sc - s64) / np.abs(s64)).max()),
+            }
+            del d
+    return rec
 
 
 def bench_joiner(args):
@@ -308,6 +417,12 @@ def main():
     ap.add_argument("--joiner-dim", type=int, default=512)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true",
+                    help="skip the parity gate (the GPU's loss and gradient for the timed workload "
+                         "against the CPU baseline's, outside the timed region)")
+    ap.add_argument("--parity-f64", action="store_true",
+                    help="also run the float64 build of the CPU restatement on the whole batch and "
+                         "report how far the GPU and the float32 reference each are from it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the library's plain copy kernel on 1 GiB (read 1 GiB + "
                          "write 1 GiB) three times, as a known-size reference for profiler "
@@ -373,19 +488,27 @@ def main():
     torch.cuda.synchronize()
 
     bufs = [pristine.clone() for _ in range(K)]
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(K + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for b in bufs:
+    marks[0].record()
+    for i, b in enumerate(bufs):
         step(b)
+        marks[i + 1].record()  # on the stream the step's kernels were launched on
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     del bufs
+    per_step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(K))
 
     out = {
         "metric": "utterances/sec fwd+bwd loss at N=32,V=500 fp32; achieved HBM GB/s vs peak",
         "value": w.N * K / elapsed, "unit": "utterances/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": 1e3 * elapsed / K, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None,
+        # spread of the K timed steps, each between two events on the launch stream
+        "step_ms": {"median": per_step_ms[K // 2] if K % 2 else
+                    0.5 * (per_step_ms[K // 2 - 1] + per_step_ms[K // 2]),
+                    "min": per_step_ms[0], "max": per_step_ms[-1]},
         "dtype": "f32" if esize == 4 else "f32 arithmetic on %s logits" % args.logits_dtype,
         "data": "synthetic",
         "config": {"workload": w.name, "N": w.N, "V": w.V, "packed_rows": w.rows,
@@ -426,18 +549,21 @@ def main():
                                                     "true" if w.from_log_softmax else "false")
         if esize == 2:
             kernel_name = "grad_flat_half_kernel"
+        traffic, traffic_source = measured_traffic(w.name, dom) if esize == 4 else (None, None)
         out["roofline"] = {"bound": "hbm", "kernel": kernel_name, "achieved": achieved,
                            "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                            "frac": achieved / HBM_PEAK_GBPS,
-                           "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, dom)) if esize == 4 else None,
+                           "traffic": traffic, "traffic_source": traffic_source,
                            "kernel_ms_per_step": kernels[dom]["ms_per_step"],
                            "launches_per_step": kernels[dom]["launches_per_step"],
                            "algorithmic_bytes_per_step": alg[dom]}
         out["kernels"] = kernels
 
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(w, pristine.float().cpu())
+        out["cpu_baseline"], ref = cpu_baseline(w, pristine.float().cpu())
         out["speedup_vs_cpu"] = out["value"] / out["cpu_baseline"]["value"]
+        if not args.no_parity:
+            out["parity"] = parity_record(w, args, pristine, targets, T, U, ref, args.parity_f64)
 
     print(json.dumps(out), flush=True)
 

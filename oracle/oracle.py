@@ -112,7 +112,9 @@ def beta(lp, logit_lengths, target_lengths, one_sym_per_frame=False):
 
 
 def gradient(logits, targets, logit_lengths, target_lengths, blank, den, alpha_, beta_,
-             one_sym_per_frame=False, out=None):
+             one_sym_per_frame=False, out=None, mag=None):
+    """``mag`` (optional array like the gradient) receives the per-entry sum of the
+    absolute values of the exponentials an entry is made of (a tolerance scale)."""
     dtype, sfx = _real(alpha_.dtype)
     logits = np.ascontiguousarray(logits, dtype=np.float32)
     targets, T, U = _i32(targets), _i32(logit_lengths), _i32(target_lengths)
@@ -120,18 +122,22 @@ def gradient(logits, targets, logit_lengths, target_lengths, blank, den, alpha_,
     getattr(lib(), "ot_oracle_gradient" + sfx)(
         _p(logits), _p(targets), ctypes.c_int32(targets.shape[1]), _p(T), _p(U),
         ctypes.c_int32(T.size), ctypes.c_int32(logits.shape[1]), ctypes.c_int32(blank),
-        _p(den), _p(alpha_), _p(beta_), ctypes.c_int32(int(one_sym_per_frame)), _p(grad))
+        _p(den), _p(alpha_), _p(beta_), ctypes.c_int32(int(one_sym_per_frame)), _p(grad),
+        _p(mag))
     return grad
 
 
 def compute_transducer_loss(logits, targets, logit_lengths, target_lengths, blank,
                             from_log_softmax, one_sym_per_frame, want_grad=True,
-                            dtype=np.float32, in_place=False, return_parts=False):
+                            dtype=np.float32, in_place=False, return_parts=False,
+                            return_magnitude=False):
     """Counterpart of ``_optimized_transducer.compute_transducer_loss``.
 
     Returns ``(scores, grad)``; scores are +log-likelihoods (cpu.cc:826).  With
     ``in_place=True`` (float32, logits input) the gradient overwrites ``logits``
-    as the reference does (cpu.cc:814).
+    as the reference does (cpu.cc:814).  With ``return_magnitude=True`` a third
+    value follows: per gradient entry, the sum of the absolute values of the
+    exponentials it is the difference of (see ``ot_oracle_gradient``).
     """
     dtype, sfx = _real(dtype)
     assert logits.dtype == np.float32 and logits.flags.c_contiguous
@@ -146,11 +152,16 @@ def compute_transducer_loss(logits, targets, logit_lengths, target_lengths, blan
             grad = logits
         else:
             grad = np.empty((rows, V), dtype=dtype)
+    mag = np.empty((rows, V), dtype=dtype) if (want_grad and return_magnitude) else None
     getattr(lib(), "ot_oracle_transducer_loss" + sfx)(
         _p(logits), _p(targets), ctypes.c_int32(targets.shape[1]), _p(T), _p(U),
         ctypes.c_int32(T.size), ctypes.c_int64(rows), ctypes.c_int32(V),
         ctypes.c_int32(blank), ctypes.c_int32(int(from_log_softmax)),
-        ctypes.c_int32(int(one_sym_per_frame)), _p(work), _p(scores), _p(scores_beta), _p(grad))
+        ctypes.c_int32(int(one_sym_per_frame)), _p(work), _p(scores), _p(scores_beta), _p(grad),
+        _p(mag))
+    if return_magnitude:
+        assert not return_parts
+        return scores, grad, mag
     if return_parts:
         parts = dict(den=work[:rows], lp=work[rows:3 * rows].reshape(rows, 2),
                      alpha=work[3 * rows:4 * rows], beta=work[4 * rows:5 * rows],

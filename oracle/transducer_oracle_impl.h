@@ -186,13 +186,18 @@ void FN(ot_oracle_beta)(const REAL *lp, const int32_t *logit_lengths,
  *                              cpu.cc:691-751
  * Evaluation order kept as in the reference: c = (alpha + loss) - den,
  * g = logit + c, then g + beta.  When REAL is float, `grad` may alias
- * `logits` (each element is read before it is written, cpu.cc:512-522). */
+ * `logits` (each element is read before it is written, cpu.cc:512-522).
+ * `mag` (may be NULL; same shape as grad, must not alias logits) receives for
+ * every entry the sum of the absolute values of the exponentials it is made
+ * of, exp(g + beta) + sub: the scale on which a rounding difference in alpha,
+ * beta or a denominator moves the entry.  It is not part of the reference; the
+ * tests derive their per-entry comparison bound from it. */
 void FN(ot_oracle_gradient)(const float *logits, const int32_t *targets,
                             int32_t targets_cols, const int32_t *logit_lengths,
                             const int32_t *target_lengths, int32_t N, int32_t V,
                             int32_t blank, const REAL *den, const REAL *alpha,
                             const REAL *beta, int32_t one_sym_per_frame,
-                            REAL *grad) {
+                            REAL *grad, REAL *mag) {
   int64_t off = 0;
   for (int32_t b = 0; b < N; ++b) {
     const int32_t T = logit_lengths[b], U1 = target_lengths[b] + 1;
@@ -206,8 +211,11 @@ void FN(ot_oracle_gradient)(const float *logits, const int32_t *targets,
         const int64_t r = off + (int64_t)t * U1 + u;
         const float *x = logits + r * (int64_t)V;
         REAL *gr = grad + r * (int64_t)V;
+        REAL *mg = mag ? mag + r * (int64_t)V : NULL;
         if (one_sym_per_frame && (u > t || t - u > diff)) {
           for (int32_t v = 0; v < V; ++v) gr[v] = 0; /* cpu.cc:582-586 */
+          if (mg)
+            for (int32_t v = 0; v < V; ++v) mg[v] = 0;
           continue;
         }
         const int32_t target_u = (u < U) ? tg[u] : -1;
@@ -232,10 +240,14 @@ void FN(ot_oracle_gradient)(const float *logits, const int32_t *targets,
             sub = 0;
             special = 0;
           }
-          if (den)
-            gr[v] = special ? R_EXP(g + BE(t, u)) - sub : R_EXP(g + BE(t, u));
-          else
+          if (den) {
+            const REAL whole = R_EXP(g + BE(t, u));
+            gr[v] = special ? whole - sub : whole;
+            if (mg) mg[v] = whole + sub;
+          } else {
             gr[v] = special ? -sub : 0;
+            if (mg) mg[v] = sub;
+          }
         }
       }
     }
@@ -258,7 +270,7 @@ void FN(ot_oracle_transducer_loss)(
     const int32_t *logit_lengths, const int32_t *target_lengths, int32_t N,
     int64_t rows, int32_t V, int32_t blank, int32_t from_log_softmax,
     int32_t one_sym_per_frame, REAL *work, REAL *scores, REAL *scores_beta,
-    REAL *grad) {
+    REAL *grad, REAL *mag) {
   REAL *den = work, *lp = work + rows, *alpha = work + 3 * rows,
        *beta = work + 4 * rows;
   if (!from_log_softmax) FN(ot_oracle_logsumexp)(logits, rows, V, den);
@@ -273,7 +285,7 @@ void FN(ot_oracle_transducer_loss)(
     FN(ot_oracle_gradient)(logits, targets, targets_cols, logit_lengths,
                            target_lengths, N, V, blank,
                            from_log_softmax ? NULL : den, alpha, beta,
-                           one_sym_per_frame, grad);
+                           one_sym_per_frame, grad, mag);
 }
 
 #undef FN

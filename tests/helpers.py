@@ -33,18 +33,36 @@ def log_softmax32(x):
     return (z - np.log(np.exp(z).sum(axis=1, keepdims=True))).astype(np.float32)
 
 
-def lattice_noise_tolerance(ref_grad, loss_per_row, k=8.0):
+# Roundings of size ulp(|log-likelihood|) that two float32 evaluations of one gradient
+# entry may differ by (see lattice_noise_tolerance).
+NOISE_K = 8.0
+
+
+def lattice_noise_tolerance(ref_grad, loss_per_row, mag, k=NOISE_K, scale=1.0):
     """Elementwise bound for comparing two fp32 evaluations of the gradient.
 
     Every entry is a difference of exponentials exp(x + c + beta) whose
     argument is a sum of terms of magnitude |loss| (cpu.cc:509-522), so two
     correct fp32 evaluations that differ by one rounding anywhere in alpha,
     beta or the denominator differ by about ulp(|loss|) in that argument, i.e.
-    by entry * ulp(|loss|).  The bound is the north-star tolerance plus k such
-    roundings of the row's own likelihood magnitude, with entries bounded by 1.
+    by ulp(|loss|) times each exponential.  ``mag`` is the sum of an entry's
+    exponentials (``return_magnitude=True`` of the oracle), so the bound scales
+    with the entry: the north-star tolerance plus k such roundings.  A wrong
+    small entry fails; an all-zero result fails wherever the entry exceeds
+    about 1e-5.  ``ref_grad`` and ``mag`` belong to the unscaled gradient;
+    ``scale`` is the factor (upstream gradient, 1/N) the compared one carries:
+    it multiplies the relative parts, and the absolute part when below 1.
     """
-    noise = k * EPS32 * np.abs(loss_per_row)[:, None]
-    return ATOL + RTOL * np.abs(ref_grad) + noise
+    noise = k * EPS32 * np.abs(loss_per_row)[:, None] * mag
+    return min(scale, 1.0) * ATOL + scale * (RTOL * np.abs(ref_grad) + noise)
+
+
+def oracle_tolerance(x, targets, T, U, blank, fls, osf, scale=1.0, k=NOISE_K):
+    """(scores, unscaled fp32 gradient, elementwise bound for `scale` x that gradient)
+    from one run of the fp32 oracle."""
+    s, g, mag = oracle.compute_transducer_loss(np.ascontiguousarray(x).copy(), targets, T, U, blank,
+                                               fls, osf, return_magnitude=True)
+    return s, g, lattice_noise_tolerance(g, per_row(s, T, U), mag, k=k, scale=scale)
 
 
 def per_row(values_per_utt, T, U):
