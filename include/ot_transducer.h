@@ -29,14 +29,19 @@ extern "C" {
 #endif
 
 #define OT_E_BAD_ARG (-1)       /* null pointer / non-positive size            */
-#define OT_E_TOO_LONG (-2)      /* max(U)+1 exceeds OT_MAX_U1                  */
+#define OT_E_TOO_LONG (-2)      /* a length exceeds what the kernels address   */
 #define OT_E_MISALIGNED (-3)    /* logits / grad not 4-byte aligned            */
 #define OT_E_TOO_LARGE (-4)     /* batch exceeds OT_STATIC_WORKSPACE_BYTES     */
 
-/* Largest U+1 the lattice kernels handle (one thread per u, one workgroup per
- * utterance and direction).  The reference's CUDA path has the same bound
- * (cuda.cu:10, cuda.cu:202). */
-#define OT_MAX_U1 1024
+/* Lattice columns (u = 0..U) one workgroup sweeps at a time, one thread per
+ * column; an utterance with more columns is swept in tiles of this width, one
+ * after the other, like the reference's CPU path loops over any U
+ * (cpu.cc:162-244; its CUDA path stops at 1024 columns, cuda.cu:10, cuda.cu:202). */
+#define OT_LATTICE_TILE 1024
+/* Largest max_u1 = max_b(U_b)+1 accepted.  What really bounds an utterance is
+ * that its cells are addressed with 32-bit byte offsets:
+ * (T_b + 1300) * (U_b + 1) < 2^29. */
+#define OT_MAX_U1 (1 << 18)
 
 /* Batch facts gathered on the device by ot_row_splits; the host-side argument
  * checks of the reference (transducer-loss.cc:49-66) need exactly these and
@@ -44,7 +49,10 @@ extern "C" {
 typedef struct ot_batch_status {
   int64_t sum_tu;          /* sum_b T_b * (U_b + 1), exact in 64 bits          */
   int32_t targets_max;     /* max over the whole (N, targets_cols) array       */
-  int32_t targets_min;     /* min over the same array                          */
+  int32_t targets_min;     /* min over the same array if that is >= 0; else
+                              min over the entries that are read, u < U_b
+                              (INT32_MAX if none): negative exactly when an
+                              entry that is read is negative                   */
   int32_t target_len_max;  /* max_b U_b                                        */
   int32_t target_len_min;  /* min_b U_b                                        */
   int32_t logit_len_max;   /* max_b T_b                                        */
@@ -100,7 +108,8 @@ int ot_log_probs_range(const float *logits, const int32_t *targets,
  * alpha, beta: (rows,) float.  scores_alpha[b] = alpha(T-1,U)+lp(T-1,U).blank,
  * scores_beta[b] = beta(0,0); both are log-likelihoods.  Cells outside the
  * band of the one-symbol-per-frame lattice (uninitialised in the reference)
- * are -inf.  max_u1 = max_b(U_b)+1 sizes the workgroup; must be <= OT_MAX_U1. */
+ * are -inf.  max_u1 = max_b(U_b)+1 sizes the workgroup; must be <= OT_MAX_U1,
+ * and every utterance must satisfy (T_b + 1300) * (U_b + 1) < 2^29. */
 int ot_alpha_beta(const float *lp, const int32_t *logit_lengths,
                   const int32_t *target_lengths, const int32_t *row_splits,
                   int32_t N, int32_t max_u1, int32_t one_sym_per_frame,

@@ -4,10 +4,14 @@
 //
 // This file only checks arguments, allocates through torch's caching allocator
 // and enqueues the C-ABI kernels of include/ot_transducer.h on torch's current
-// HIP stream.  There is no CPU implementation behind it: CPU tensors are
-// checked like the reference checks them and then rejected.
+// HIP stream.  There is no CPU implementation behind it: CPU tensors, which the
+// reference hands to ComputeTransducerLossCpu (transducer-loss.cc:68-74), are
+// checked like the reference checks them, copied to the current HIP device,
+// computed there and copied back (the gradient of logits input into the caller's
+// logits storage, as cpu.cc:814 aliases it).
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/hip/HIPFunctions.h>
 #include <hip/hip_runtime_api.h>
 #include <torch/extension.h>
 
@@ -190,7 +194,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
 
   if (logits.device().type() == torch::kCPU) {
     // Same checks as the reference makes before it dispatches on the device
-    // (transducer-loss.cc:49-71); then refuse: this build has no CPU path.
+    // (transducer-loss.cc:49-71), on the host tensors.
     TORCH_CHECK(N > 0, "logit_lengths must not be empty");
     const int64_t sum_all_TU =
         (logit_lengths.to(torch::kLong) * (target_lengths.to(torch::kLong) + 1)).sum().item<int64_t>();
@@ -199,10 +203,32 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
     check_batch_values(logits, targets, sum_all_TU, targets_max, target_len_max, blank);
     torch::checkDeviceType(checked_from, {logits, targets, logit_lengths, target_lengths},
                            torch::kCPU);
-    throw std::runtime_error(
-        "optimized_transducer_amd computes on MI355X (HIP) only and has no CPU "
-        "implementation; move logits, targets, logit_lengths and target_lengths "
-        "to a HIP device (tensor.cuda()).");
+    TORCH_CHECK(!defer, "defer_gradient needs logits on a HIP device");
+    TORCH_CHECK(!have_den || denominators->device().type() == torch::kCPU,
+                "denominators must be on the device of logits");
+    // The reference computes these on the host (ComputeTransducerLossCpu, cpu.cc:754-827).
+    // This build computes on the GPU only: stage the batch through the current HIP device.
+    if (!torch::cuda::is_available())
+      throw std::runtime_error(
+          "optimized_transducer_amd: CPU tensors are computed on a HIP device (there is no CPU "
+          "implementation), and no HIP device is available");
+    const torch::Device dev(torch::kCUDA, c10::hip::current_device());
+    torch::Tensor dev_logits = logits.detach().to(dev);
+    if (logits.requires_grad()) dev_logits.requires_grad_(true);
+    torch::optional<torch::Tensor> dev_den;
+    if (have_den) dev_den = denominators->to(dev);
+    torch::Tensor dev_loss;
+    auto out = compute_impl(dev_logits, targets.to(dev), logit_lengths.to(dev),
+                            target_lengths.to(dev), blank, from_log_softmax, one_sym_per_frame,
+                            grad_scale, nullptr, dev_den, reduced_loss ? &dev_loss : nullptr);
+    if (reduced_loss) *reduced_loss = dev_loss.cpu();
+    torch::Tensor scores = out.first.cpu();
+    if (!out.second.has_value()) return {scores, torch::nullopt};
+    // cpu.cc:803: a new tensor for log-softmax input
+    if (from_log_softmax) return {scores, out.second->cpu()};
+    // cpu.cc:814: for logits input the gradient IS the caller's logits buffer
+    logits.detach().copy_(*out.second);
+    return {scores, logits};
   }
 
   torch::checkAllSameGPU(checked_from,
@@ -211,7 +237,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   TORCH_CHECK(targets.size(0) == N, "targets.size(0) is ", targets.size(0),
               " but there are ", N, " utterances");
   TORCH_CHECK(rows > 0 && V > 0, "logits must not be empty");
-  TORCH_CHECK(rows <= INT32_MAX && N < INT32_MAX && V <= INT32_MAX && S < OT_MAX_U1 * 64,
+  TORCH_CHECK(rows <= INT32_MAX && N < INT32_MAX && V <= INT32_MAX && S < OT_MAX_U1,
               "tensor sizes exceed what 32-bit row offsets can address");
   if (have_den) {
     TORCH_CHECK(!from_log_softmax, "denominators belong to logits input (from_log_softmax=False)");
@@ -320,7 +346,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
   // The host's wake-up and its remaining launches then hide behind it even when the
   // first kernel is the short gather of log-softmax input.
   torch::Tensor scores = torch::empty({N}, logits.options().dtype(torch::kFloat));
-  const bool early_lattice = blank_ok && !overlap && S + 1 <= OT_MAX_U1;
+  const bool early_lattice = blank_ok && !overlap;
   if (early_lattice) {
     ScopedTimer timer("alpha_beta", stream);
     OT_CHECK(ot_alpha_beta_guarded(lp, p_T, p_U, row_splits, (int32_t)N, (int32_t)S + 1,
@@ -334,15 +360,15 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
 
   check_batch_values(logits, targets, st.sum_tu, S > 0 ? (int64_t)st.targets_max : INT32_MIN,
                      st.target_len_max, blank);
-  // beyond the reference (which has undefined behaviour for these)
-  TORCH_CHECK(S == 0 || st.targets_min >= 0, "targets.min() is ", st.targets_min,
-              ". Expect targets.min() >= 0");
+  // beyond the reference (which has undefined behaviour for these): a negative id among the
+  // entries that are read, u < target_lengths[b]; padding behind them is never read
+  // (kernels.cu:49-50) and may hold anything below logits.size(1), e.g. -1
+  TORCH_CHECK(S == 0 || st.targets_min >= 0, "targets.min() over the valid entries is ",
+              st.targets_min, ". Expect targets >= 0");
   TORCH_CHECK(st.logit_len_min >= 1 && st.target_len_min >= 0,
               "Expect logit_lengths >= 1 and target_lengths >= 0, but the minima are ",
               st.logit_len_min, " and ", st.target_len_min);
   const int32_t max_u1 = st.target_len_max + 1;
-  TORCH_CHECK(max_u1 <= OT_MAX_U1, "target_lengths.max() + 1 is ", max_u1,
-              ", which exceeds the supported ", OT_MAX_U1);
   // the lattice kernel addresses one utterance's cells with 32-bit byte offsets
   TORCH_CHECK(((int64_t)st.logit_len_max + 1300) * max_u1 < ((int64_t)1 << 29),
               "an utterance with T = ", st.logit_len_max, " and up to ", max_u1,

@@ -114,6 +114,23 @@ __global__ __launch_bounds__(kPrepThreads) void prepare_kernel(
     atomicMax(&s_red[4], tmax); atomicMin(&s_red[5], tmin);
   }
   __syncthreads();
+  // The minimum that matters is the one over the entries the kernels read, u < U_b
+  // (padding behind them may be -1).  Only a batch whose whole-array minimum is
+  // negative needs the second, row-aware pass.
+  if (s_red[1] < 0) {
+    __syncthreads();
+    if (tid == 0) s_red[1] = INT32_MAX;
+    __syncthreads();
+    int vmin = INT32_MAX;
+    for (int b = tid / kWave; b < N; b += kPrepThreads / kWave) {
+      const int U = min(target_lengths[b], targets_cols);
+      for (int u = tid & (kWave - 1); u < U; u += kWave)
+        vmin = min(vmin, targets[(long long)b * targets_cols + u]);
+    }
+    for (int ofs = kWave / 2; ofs > 0; ofs >>= 1) vmin = min(vmin, __shfl_xor(vmin, ofs, kWave));
+    if ((tid & (kWave - 1)) == 0) atomicMin(&s_red[1], vmin);
+    __syncthreads();
+  }
   if (tid == 0) {
     status->sum_tu = s_total;
     status->targets_max = s_red[0];
@@ -311,30 +328,40 @@ __global__ __launch_bounds__(kBlock) void lse_gather_kernel(
 // (none at all for a single wave).  The lp values do not depend on the
 // recursion and are fetched kChunk steps ahead.
 // ---------------------------------------------------------------------------
-constexpr int kMaxDpWaves = OT_MAX_U1 / kWave;
+constexpr int kMaxDpWaves = OT_LATTICE_TILE / kWave;
 constexpr int kChunk = 16;  // steps between barriers
 constexpr int kLag = kChunk;
 constexpr int kRing = 64;   // >= 2*kChunk + 2 slots per wave boundary
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-template <bool BETA, bool OSF, bool MULTI>
+// TILED: the workgroup's threads cover the OT_LATTICE_TILE columns that start at u0, and
+// the lattice is swept tile by tile (lattice_tiles).  The column next to the tile on the
+// side the recursion comes from belongs to a tile that is already complete in `out`; the
+// tile's edge lane takes its neighbour values from there, one load per step, fetched a
+// chunk at a time like the values that cross a wave boundary.
+template <bool BETA, bool OSF, bool MULTI, bool TILED = false>
 __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int T, int U,
                                               int64_t row0, float *__restrict__ out,
                                               float *__restrict__ score,
-                                              float (*s_ring)[kRing + kChunk]) {
-  const int u = threadIdx.x;
-  const int lane = u & (kWave - 1), wave = u / kWave;
+                                              float (*s_ring)[kRing + kChunk], int u0 = 0) {
+  static_assert(MULTI || !TILED, "a tiled sweep has several waves");
+  const int u = u0 + (int)threadIdx.x;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int U1 = U + 1;
-  const int wlast = U / kWave;  // wave that owns u == U
-  const int nsteps = (OSF ? T : T + U) + (MULTI ? wlast * kLag : 0);
-  const bool column = u < U1;
+  // the sweep's columns are [u0, u_top]
+  const int u_top = TILED ? min(U, u0 + OT_LATTICE_TILE - 1) : U;
+  const int wlast = (u_top - u0) / kWave;  // wave that owns u_top
+  const int nsteps = (OSF ? T : T + (u_top - u0)) + (MULTI ? wlast * kLag : 0);
+  const bool column = u <= u_top;
   // (unsigned)(t - u) < band  <=>  u <= t && t - u <= T-1-U   (never, if infeasible)
   const unsigned band = (unsigned)(max(T - 1 - U, -1) + 1);
 
   int delay;
-  if (BETA) delay = (OSF ? 0 : U - u) + (MULTI ? (wlast - wave) * kLag : 0);
-  else delay = (OSF ? 0 : u) + (MULTI ? wave * kLag : 0);
+  if (BETA) delay = (OSF ? 0 : u_top - u) + (MULTI ? (wlast - wave) * kLag : 0);
+  else delay = (OSF ? 0 : u - u0) + (MULTI ? wave * kLag : 0);
+  // does the recursion enter this tile from a column of another tile?
+  const bool gsrc = TILED && (BETA ? u_top < U : u0 > 0);
 
   // This utterance's slice as raw buffers: a cell index outside [0, T*U1)
   // (t < 0, t >= T, or the forced offset of a thread without a column) reads
@@ -399,6 +426,26 @@ __device__ __forceinline__ void lattice_sweep(const float *__restrict__ lp, int 
       const float v = s_ring[src_ok][s & (kRing - 1)];
       ering = (has_src && ering_step < kChunk && s >= 0) ? v : OT_NEG_INF;
       ring_wr = ring_dst + (n & ring_mask);  // n is a multiple of kChunk: no wrap inside a chunk
+      if (TILED && gsrc && wave == (BETA ? wlast : 0)) {
+        // The tile's edge column (delay 0) is in row tc at step n + ering_step; what the
+        // neighbouring column hands over then is, for alpha, alpha + sym of the cell the
+        // symbol arc comes from (same row; the row before on the one-symbol-per-frame
+        // lattice) and, for beta, beta of the cell the symbol arc leads to.  Rows outside
+        // the lattice hand over -inf.
+        const int sc = n + ering_step;
+        const int tc = BETA ? (T - 1 - sc) : sc;
+        const int te = OSF ? (BETA ? tc + 1 : tc - 1) : tc;
+        const int ue = BETA ? u_top + 1 : u0 - 1;
+        const bool ok = ering_step < kChunk && (unsigned)te < (unsigned)T;
+        const unsigned cell = ok ? (unsigned)(te * U1 + ue) : 0x10000000u;
+        // sc0 sc1: served by the device-wide cache, where the earlier tile's stores are
+        float e = __builtin_bit_cast(
+            float, __builtin_amdgcn_raw_buffer_load_b32(out_buf, cell * 4u, 0, 17));
+        if (!BETA)
+          e += __builtin_bit_cast(
+              float, __builtin_amdgcn_raw_buffer_load_b32(lp_buf, cell * 8u + 4u, 0, 0));
+        ering = ok ? e : OT_NEG_INF;
+      }
     }
 #pragma unroll
     for (int i = 0; i < kChunk; ++i) {
@@ -576,12 +623,12 @@ __device__ __forceinline__ void lattice_sweep_staged(const float *__restrict__ l
 // A lattice kernel that is launched before the host has seen the batch facts checks
 // what its memory safety rests on itself and does nothing otherwise (guard_n = N, or 0
 // for a launch after validation): the rows of the batch add up to the size of the
-// arrays, every utterance has T >= 1 and 0 <= U < the workgroup's columns, and its cells
-// fit 32-bit byte offsets.
+// arrays, every utterance has T >= 1 and 0 <= U < the columns the launch was sized for,
+// and its cells fit 32-bit byte offsets.
 __device__ __forceinline__ bool lattice_guard_ok(const int32_t *__restrict__ row_splits, int guard_n,
-                                                 int64_t guard_rows, int T, int U) {
+                                                 int64_t guard_rows, int T, int U, int max_u1) {
   if (guard_n <= 0) return true;
-  return (int64_t)row_splits[guard_n] == guard_rows && T >= 1 && U >= 0 && U < (int)blockDim.x &&
+  return (int64_t)row_splits[guard_n] == guard_rows && T >= 1 && U >= 0 && U < max_u1 &&
          ((int64_t)T + 1300) * ((int64_t)U + 1) < ((int64_t)1 << 29);
 }
 
@@ -596,7 +643,7 @@ __global__ __launch_bounds__(THREADS) void alpha_beta_staged_kernel(
   extern __shared__ __attribute__((aligned(16))) float s_stage[];
   const int b = utt_begin + blockIdx.x;
   const int T = logit_lengths[b], U = target_lengths[b];
-  if (!lattice_guard_ok(row_splits, guard_n, guard_rows, T, U)) return;
+  if (!lattice_guard_ok(row_splits, guard_n, guard_rows, T, U, (int)blockDim.x)) return;
   const int64_t row0 = row_splits[b];
   if (blockIdx.y == 0)
     lattice_sweep_staged<false, G>(lp, T, U, row0, alpha, scores_alpha + b, s_ring, s_stage);
@@ -604,22 +651,48 @@ __global__ __launch_bounds__(THREADS) void alpha_beta_staged_kernel(
     lattice_sweep_staged<true, G>(lp, T, U, row0, beta, scores_beta + b, s_ring, s_stage);
 }
 
-template <bool OSF, bool MULTI>
-__global__ __launch_bounds__(OT_MAX_U1) void alpha_beta_kernel(
+// One sweep per tile of OT_LATTICE_TILE columns, in the order of the recursion (alpha:
+// ascending u, beta: descending).  A tile reads the finished neighbouring column from
+// `out`, so the workgroup's stores are made visible and all its waves meet between tiles.
+template <bool BETA, bool OSF>
+__device__ __forceinline__ void lattice_tiles(const float *__restrict__ lp, int T, int U,
+                                              int64_t row0, float *__restrict__ out,
+                                              float *__restrict__ score,
+                                              float (*s_ring)[kRing + kChunk]) {
+  const int ntiles = U / OT_LATTICE_TILE + 1;
+  for (int k = 0; k < ntiles; ++k) {
+    if (k) {
+      __threadfence();
+      __syncthreads();
+    }
+    const int tile = BETA ? ntiles - 1 - k : k;
+    lattice_sweep<BETA, OSF, true, true>(lp, T, U, row0, out, score, s_ring,
+                                         tile * OT_LATTICE_TILE);
+  }
+}
+
+template <bool OSF, bool MULTI, bool TILED>
+__global__ __launch_bounds__(OT_LATTICE_TILE) void alpha_beta_kernel(
     const float *__restrict__ lp, const int32_t *__restrict__ logit_lengths,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
     int utt_begin, float *__restrict__ alpha, float *__restrict__ beta,
-    float *__restrict__ scores_alpha, float *__restrict__ scores_beta, int guard_n,
+    float *__restrict__ scores_alpha, float *__restrict__ scores_beta, int max_u1, int guard_n,
     int64_t guard_rows) {
   __shared__ float s_ring[MULTI ? kMaxDpWaves : 1][kRing + kChunk];
   const int b = utt_begin + blockIdx.x;
   const int T = logit_lengths[b], U = target_lengths[b];
-  if (!lattice_guard_ok(row_splits, guard_n, guard_rows, T, U)) return;
+  if (!lattice_guard_ok(row_splits, guard_n, guard_rows, T, U, max_u1)) return;
   const int64_t row0 = row_splits[b];
-  if (blockIdx.y == 0)
+  if (TILED) {
+    if (blockIdx.y == 0)
+      lattice_tiles<false, OSF>(lp, T, U, row0, alpha, scores_alpha + b, s_ring);
+    else
+      lattice_tiles<true, OSF>(lp, T, U, row0, beta, scores_beta + b, s_ring);
+  } else if (blockIdx.y == 0) {
     lattice_sweep<false, OSF, MULTI>(lp, T, U, row0, alpha, scores_alpha + b, s_ring);
-  else
+  } else {
     lattice_sweep<true, OSF, MULTI>(lp, T, U, row0, beta, scores_beta + b, s_ring);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -990,11 +1063,13 @@ static int launch_alpha_beta(const float *lp, const int32_t *logit_lengths,
   if (max_u1 > OT_MAX_U1) return OT_E_TOO_LONG;
   if (utt_begin == utt_end) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int threads = ((max_u1 + kWave - 1) / kWave) * kWave;
+  // more columns than a workgroup has threads: column tiles, one after the other
+  const bool tiled = max_u1 > OT_LATTICE_TILE;
+  const int threads = tiled ? OT_LATTICE_TILE : ((max_u1 + kWave - 1) / kWave) * kWave;
   const dim3 grid((unsigned)(utt_end - utt_begin), 2), block((unsigned)threads);
   const bool multi = threads > kWave;
   const int nwaves = threads / kWave;
-  if (!one_sym_per_frame && nwaves >= 3) {
+  if (!one_sym_per_frame && nwaves >= 3 && !tiled) {
     // staging rings: (8 + 4) bytes per lane and group row
     const int G = nwaves <= 4 ? 16 : nwaves <= 9 ? 8 : 4;
     const size_t lds = (size_t)nwaves * G * kWave * 12;
@@ -1008,14 +1083,18 @@ static int launch_alpha_beta(const float *lp, const int32_t *logit_lengths,
 #undef OT_LAUNCH_DPS
     return launch_status();
   }
-#define OT_LAUNCH_DP(OSF_, MULTI_)                                                              \
-  hipLaunchKernelGGL((alpha_beta_kernel<OSF_, MULTI_>), grid, block, 0, s, lp, logit_lengths,   \
-                     target_lengths, row_splits, utt_begin, alpha, beta, scores_alpha, scores_beta, \
-                     guard_n, guard_rows)
+#define OT_LAUNCH_DP(OSF_, MULTI_, TILED_)                                                      \
+  hipLaunchKernelGGL((alpha_beta_kernel<OSF_, MULTI_, TILED_>), grid, block, 0, s, lp,          \
+                     logit_lengths, target_lengths, row_splits, utt_begin, alpha, beta,         \
+                     scores_alpha, scores_beta, tiled ? max_u1 : threads, guard_n, guard_rows)
   if (one_sym_per_frame) {
-    if (multi) OT_LAUNCH_DP(true, true); else OT_LAUNCH_DP(true, false);
+    if (tiled) OT_LAUNCH_DP(true, true, true);
+    else if (multi) OT_LAUNCH_DP(true, true, false);
+    else OT_LAUNCH_DP(true, false, false);
   } else {
-    if (multi) OT_LAUNCH_DP(false, true); else OT_LAUNCH_DP(false, false);
+    if (tiled) OT_LAUNCH_DP(false, true, true);
+    else if (multi) OT_LAUNCH_DP(false, true, false);
+    else OT_LAUNCH_DP(false, false, false);
   }
 #undef OT_LAUNCH_DP
   return launch_status();
@@ -1332,7 +1411,7 @@ const char *ot_error_string(int code) {
   switch (code) {
     case 0: return "success";
     case OT_E_BAD_ARG: return "ot: null pointer, non-positive size or out-of-range argument";
-    case OT_E_TOO_LONG: return "ot: max(target_lengths)+1 exceeds OT_MAX_U1";
+    case OT_E_TOO_LONG: return "ot: a length exceeds what the kernels address (OT_MAX_U1 lattice columns)";
     case OT_E_MISALIGNED: return "ot: float buffer is not 4-byte aligned";
     case OT_E_TOO_LARGE:
       return "ot: the batch needs more workspace than OT_STATIC_WORKSPACE_BYTES; use "

@@ -121,6 +121,14 @@ class TransducerLossFunction(torch.autograd.Function):
         # Hand autograd a fresh alias of the gradient buffer and drop ours: when
         # `logits` is a leaf, autograd then adopts the buffer as logits.grad
         # instead of cloning (rows, V) floats because others still hold it.
+        # The buffer is then autograd's (it may accumulate into it), so a second
+        # backward through the same graph (retain_graph=True), which the reference
+        # answers with the same tensor again (transducer_loss.py:160-162), is refused.
+        if ctx.grad is None:
+            raise RuntimeError(
+                "backward through transducer_loss runs once: the gradient buffer was handed "
+                "to autograd by the first backward (call transducer_loss again instead of "
+                "retain_graph=True)")
         grad = ctx.grad.detach()
         ctx.grad = None
         if (
@@ -191,13 +199,16 @@ def transducer_loss(
     """Transducer loss of a packed batch.
 
     Args:
-      logits: (sum_i T_i * (U_i + 1), V) float32, contiguous, on a HIP device:
+      logits: (sum_i T_i * (U_i + 1), V) float32, contiguous, on a HIP device
+        (CPU tensors are accepted like in the reference: they are copied to the
+        current HIP device, computed there and copied back):
         utterance i's (T_i, U_i + 1, V) joiner output reshaped to 2-D, all
         utterances concatenated, no padding.  Output of ``nn.Linear`` when
         ``from_log_softmax`` is False (then it is OVERWRITTEN with its gradient
         if it requires grad), output of ``log_softmax`` otherwise.
-      targets: (N, max_i U_i) int32, not prepended with blank; every entry,
-        padding included, must be in [0, V).
+      targets: (N, max_i U_i) int32, not prepended with blank; every entry
+        must be below V (the reference checks the padding too), the entries
+        u < U_i must not be negative.
       logit_lengths: (N,) int32, T_i.
       target_lengths: (N,) int32, U_i.
       blank: ID of the blank symbol, 0 <= blank < V.

@@ -129,6 +129,10 @@ WIDE = [  # (T, U) per utterance: 2..16 waves' worth of columns, mixed with shor
     ("nine_waves", [(33, 575), (100, 577), (5, 70)]),
     ("ten_waves", [(25, 600), (1, 639), (80, 129)]),
     ("sixteen_waves", [(40, 1023), (3, 700), (17, 1000), (30, 63)]),
+    # more columns than a workgroup has threads: tiles of 1024 columns, one after the other
+    # (U + 1 = 1500 and 3000; 1024 and 1025 columns sit on the tile boundary)
+    ("tiles_1500", [(60, 1499), (40, 1023), (9, 1024), (30, 63), (1, 1200)]),
+    ("tiles_3000", [(120, 2999), (35, 2047), (7, 2048), (50, 100)]),
 ]
 
 

@@ -43,8 +43,8 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_device():
     assert L.ot_log_probs(null, null, null, null, i32(1), i32(0), i64(4), i32(8), i32(0), i32(0),
                           null, null, null) == -1
     one = ctypes.c_void_p(16)  # never dereferenced: the size checks fail first
-    assert L.ot_alpha_beta(one, one, one, one, i32(1), i32(2000), i32(0), one, one, one, one,
-                           null) == -2  # OT_E_TOO_LONG
+    assert L.ot_alpha_beta(one, one, one, one, i32(1), i32((1 << 18) + 1), i32(0), one, one, one,
+                           one, null) == -2  # OT_E_TOO_LONG
     assert L.ot_log_probs(one, one, one, one, i32(1), i32(1), i64(4), i32(8), i32(9), i32(0), one,
                           one, null) == -1  # blank >= V
     assert L.ot_gradient(null, null, null, null, null, null, null, null, null, i32(1), i32(0),
@@ -140,12 +140,25 @@ def test_argument_checks_raise_like_the_reference(name):
         assert msg == want
 
 
-def test_valid_cpu_tensors_are_refused_not_computed():
+@pytest.mark.skipif(torch.cuda.is_available(), reason="with a GPU, CPU tensors are computed on it")
+def test_valid_cpu_tensors_fail_loudly_without_a_hip_device():
+    # CPU tensors are staged through the GPU (tests/test_gpu_drop_in.py); without one there
+    # is nothing to fall back to, and the call says so instead of computing on the host
     import optimized_transducer_amd as ot
     msg = _message(ot._optimized_transducer.compute_transducer_loss, _good())
-    assert "no CPU implementation" in msg
-    with pytest.raises(RuntimeError):
+    assert "no CPU implementation" in msg and "no HIP device" in msg
+    with pytest.raises(RuntimeError, match="no HIP device"):
         ot.transducer_loss(**{k: v for k, v in _good().items()}, reduction="sum")
+
+
+def test_the_reference_import_line_works():
+    # optimized_transducer/python/optimized_transducer/__init__.py:11
+    import optimized_transducer
+    import optimized_transducer_amd as ot
+    assert optimized_transducer.transducer_loss is ot.transducer_loss
+    assert optimized_transducer.TransducerLoss is ot.TransducerLoss
+    from optimized_transducer.transducer_loss import TransducerLossFunction
+    assert TransducerLossFunction is ot.TransducerLossFunction
 
 
 def test_reduction_none_is_rejected_like_the_reference():
