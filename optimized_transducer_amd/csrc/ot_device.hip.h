@@ -198,6 +198,19 @@ __device__ __forceinline__ Cell decode_row(const BlockUtterances &bu, int64_t ro
   return c;
 }
 
+// Workgroups are handed to the chip's 8 XCDs (each with its own L2) in turn: workgroup i
+// runs on XCD i % 8.  This maps workgroup i to the logical block it should work on such
+// that every XCD takes runs of `run` consecutive logical blocks (inside groups of 8 * run
+// blocks; the last, partial group keeps the identity), so that small per-row data shared by
+// neighbouring blocks is fetched into one L2 instead of several.
+__device__ __forceinline__ unsigned xcd_run_block(unsigned bid, unsigned nblocks, unsigned run) {
+  const unsigned group = 8u * run;
+  const unsigned g = bid / group;
+  if (run <= 1u || (g + 1u) * group > nblocks) return bid;
+  const unsigned r = bid - g * group;
+  return g * group + (r & 7u) * run + (r >> 3);
+}
+
 // first column index of a row's gradient coefficients that marks an all-zero row
 constexpr int kZeroRow = -2;
 

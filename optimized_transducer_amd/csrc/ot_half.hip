@@ -16,6 +16,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "ot_device.hip.h"
 #include "ot_transducer.h"
 
@@ -226,29 +228,36 @@ __global__ __launch_bounds__(kBlock) void lse_gather_half_flat_kernel(
     issue_span(base + kWavesPerBlock * G);  // past row_end: all zeros, never used
     float x[K][4];
     float cm = OT_NEG_INF;
+    // two elements of -inf in the array's type: slots past the row's end are replaced by
+    // them before the conversion (rows past row_end compute values nobody uses)
+    constexpr unsigned kNegInfPair = std::is_same<E, BF16>::value ? 0xff80ff80u : 0xfc00fc00u;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
       const int j = k * L + sub;
-      // always inside the wave's buffer; slots past the row are masked
-      const uint2 r = *reinterpret_cast<const uint2 *>(stage + (g * nvec + j) * 8);
-      const bool keep = (j < nvec) & active;
+      // always inside the wave's buffer
+      uint2 r = *reinterpret_cast<const uint2 *>(stage + (g * nvec + j) * 8);
+      const bool keep = j < nvec;
+      r.x = keep ? r.x : kNegInfPair;
+      r.y = keep ? r.y : kNegInfPair;
       x[k][0] = to_float<E>((unsigned short)(r.x & 0xffffu));
       x[k][1] = to_float<E>((unsigned short)(r.x >> 16));
       x[k][2] = to_float<E>((unsigned short)(r.y & 0xffffu));
       x[k][3] = to_float<E>((unsigned short)(r.y >> 16));
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        x[k][e] = keep ? x[k][e] : OT_NEG_INF;
-        cm = fmaxf(cm, x[k][e]);
-      }
+      for (int e = 0; e < 4; ++e) cm = fmaxf(cm, x[k][e]);
     }
     float m = group_allreduce<L>(cm, MaxOp());
     if (__builtin_isinf(m)) m = 0.f;  // as ATen's logsumexp does for an all -inf / +inf row
+    // exp(x - m) = 2^(x * log2(e) - m * log2(e)): one fused multiply-add per element.  The
+    // rounding of m * log2(e) shifts every term of the row by the same factor, at most
+    // half an ulp of m in the logarithm of the sum, i.e. less than one ulp of the result.
+    constexpr float kLog2e = 1.44269502162933349609375f;
+    const float mshift = -m * kLog2e;
     float acc = 0.f;
 #pragma unroll
     for (int k = 0; k < K; ++k)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc += exp_fast(x[k][e] - m);
+      for (int e = 0; e < 4; ++e) acc += __builtin_amdgcn_exp2f(__builtin_fmaf(x[k][e], kLog2e, mshift));
     const float d = logf(group_allreduce<L>(acc, SumOp())) + m;
 
     if (active) {
@@ -426,18 +435,35 @@ __device__ __forceinline__ void grad_piece(const float *x, float *y, const float
       }
     }
   } else {
-    const bool zero = ci.x == kZeroRow;
-    const float shift = f.x + f.y;
+    // exp(x + shift) = 2^(x * log2(e) + shift * log2(e)): one fused multiply-add and one
+    // hardware 2^x per element
+    constexpr float kLog2e = 1.44269502162933349609375f;
+    const float shift = (f.x + f.y) * kLog2e;
+    if (ci.x == kZeroRow) {  // exact zeros whatever the logits hold
 #pragma unroll
-    for (int e = 0; e < S; ++e) {
-      const float v = exp_fast(x[e] + shift);
-      y[e] = zero ? 0.f : v;
+      for (int e = 0; e < S; ++e) y[e] = 0.f;
+      return;
     }
-    if (special) {
 #pragma unroll
-      for (int e = 0; e < S; ++e) {
-        if (d1 == (unsigned)e) y[e] = exp_any((x[e] + f.x) + f.y) - exp_any((x[e] + f.x) + f.z);
-        if (d2 == (unsigned)e) y[e] = exp_any((x[e] + f.x) + f.y) - exp_any((x[e] + f.x) + f.w);
+    for (int e = 0; e < S; ++e) y[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[e], kLog2e, shift));
+    if (special) {
+      // at most one element per special column: pick it, evaluate the two accurate
+      // exponentials once, and put the difference back
+      if (d1 < (unsigned)S) {
+        float xe = x[0];
+#pragma unroll
+        for (int e = 1; e < S; ++e) xe = (d1 == (unsigned)e) ? x[e] : xe;
+        const float v = exp_any((xe + f.x) + f.y) - exp_any((xe + f.x) + f.z);
+#pragma unroll
+        for (int e = 0; e < S; ++e) y[e] = (d1 == (unsigned)e) ? v : y[e];
+      }
+      if (d2 < (unsigned)S) {
+        float xe = x[0];
+#pragma unroll
+        for (int e = 1; e < S; ++e) xe = (d2 == (unsigned)e) ? x[e] : xe;
+        const float v = exp_any((xe + f.x) + f.y) - exp_any((xe + f.x) + f.w);
+#pragma unroll
+        for (int e = 0; e < S; ++e) y[e] = (d2 == (unsigned)e) ? v : y[e];
       }
     }
     if (scale != 1.f) {
@@ -468,7 +494,14 @@ __global__ __launch_bounds__(kBlock) void grad_flat_half_kernel(
   const float factor = device_factor ? *device_factor : 1.f;
   if (!FLS) scale *= factor;
   constexpr int kPerBlock = kHalfGradUnroll * kBlock * kHalfWide;  // elements per workgroup
-  const int64_t base = (int64_t)blockIdx.x * kPerBlock;
+  // Every XCD takes runs of 16 consecutive workgroups' worth of the array (128 KB): the
+  // 24-byte row coefficients, which several neighbouring workgroups share, are then fetched
+  // into one L2 instead of up to eight (2-byte rows are half as long, so the eightfold
+  // fetch weighs twice what it does for float32 logits), +4-6 % for the in-place stream.
+  // Runs of 8 help less, 32 and runs that are no power of two not at all; the float32
+  // kernel loses 2-6 % with any such mapping.
+  const unsigned lblock = xcd_run_block(blockIdx.x, gridDim.x, 16u);
+  const int64_t base = (int64_t)lblock * kPerBlock;
   // base / V through a double reciprocal (exact below 2^53) and one correction step
   int64_t row_base = (int64_t)((double)base * inv_v_d);
   {
@@ -526,7 +559,7 @@ __global__ __launch_bounds__(kBlock) void grad_flat_half_kernel(
                                            kAuxStreamStore);
   }
   // the last total % 8 elements (a multiple of S), S at a time
-  if (S < kHalfWide && blockIdx.x == gridDim.x - 1) {
+  if (S < kHalfWide && lblock == gridDim.x - 1) {
     const int64_t elem = wide_end + (int64_t)threadIdx.x * S;
     if (elem < total) {
       float xs[S], ys[S];

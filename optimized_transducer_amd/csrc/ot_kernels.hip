@@ -870,13 +870,24 @@ __global__ __launch_bounds__(grad_block(FLS, VEC)) void grad_flat_kernel(
       const bool zero = ci.x == kZeroRow;
 #pragma unroll
       for (int e = 0; e < VEC; ++e) y.v[e] = zero ? 0.f : exp_any((x[k].v[e] + f.x) + f.y);
+      // at most one element of the unit per special column: pick it and evaluate the
+      // subtracted exponential once
       const unsigned d1 = (unsigned)(ci.x - col0[k]), d2 = (unsigned)(ci.y - col0[k]);
-      if (d1 < (unsigned)VEC || d2 < (unsigned)VEC) {
+      if (d1 < (unsigned)VEC) {
+        float xe = x[k].v[0];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          if (d1 == (unsigned)e) y.v[e] -= exp_any((x[k].v[e] + f.x) + f.z);
-          if (d2 == (unsigned)e) y.v[e] -= exp_any((x[k].v[e] + f.x) + f.w);
-        }
+        for (int e = 1; e < VEC; ++e) xe = (d1 == (unsigned)e) ? x[k].v[e] : xe;
+        const float sub = exp_any((xe + f.x) + f.z);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) y.v[e] = (d1 == (unsigned)e) ? y.v[e] - sub : y.v[e];
+      }
+      if (d2 < (unsigned)VEC) {
+        float xe = x[k].v[0];
+#pragma unroll
+        for (int e = 1; e < VEC; ++e) xe = (d2 == (unsigned)e) ? x[k].v[e] : xe;
+        const float sub = exp_any((xe + f.x) + f.w);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) y.v[e] = (d2 == (unsigned)e) ? y.v[e] - sub : y.v[e];
       }
       if (scale != 1.f) {
 #pragma unroll
