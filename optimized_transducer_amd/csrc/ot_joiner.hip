@@ -211,11 +211,12 @@ constexpr int kSlabLanes = 16;      // lanes across the columns of a slab: 16 x 
 constexpr int kSlabLanesHalf = 32;  // 32 x 8 bytes of a 2-byte row (256 contiguous bytes either way)
 
 // One workgroup: utterance b = blockIdx.z, frames [t0, t0 + 16), columns
-// [slab*16*VEC, (slab+1)*16*VEC).  Thread (phase, lane): columns lane*VEC.., and
-// the positions u = phase, phase + 16, ...  For one u it loads the 16 frames'
-// values (16 independent loads), adds them up for the decoder and into 16
-// per-frame accumulators for the encoder.  The encoder sums of the workgroup's
-// threads are then added through DPP/LDS in a fixed order.
+// [slab*SL*VEC, (slab+1)*SL*VEC).  Thread (phase, half, lane): columns lane*VEC.., the
+// positions u = phase, phase + P, ... and 8 of the tile's 16 frames.  For one u it loads
+// its 8 frames' values (8 independent loads), adds them up for the decoder (the two
+// halves meet through one cross-lane exchange) and into 8 per-frame accumulators for
+// the encoder.  The encoder sums of the workgroup's threads are then added through
+// DPP/LDS in a fixed order.
 // VEC elements of the incoming gradient: float32 (G = float) or a 2-byte type.  Loading
 // and widening are two steps so that a thread's 16 loads are all issued before the
 // first value is used.
@@ -248,6 +249,16 @@ template <int VEC> struct GradIO<float, VEC> {
 };
 
 // G: element type of grad_out (float, F16 or BF16); everything else is float32.
+//
+// Thread (phase, half, lane): columns lane*VEC.., the positions u = phase, phase + P, ...
+// (P = 128 / SL phases per workgroup), and the 8 frames half*8 .. half*8+7 of the tile.
+// The two halves of a position sit in one wave, SL lanes apart, and meet through one
+// cross-lane exchange per position.  With all 16 frames in one thread the kernel needs
+// 170-250 registers (16 values in flight, 16 accumulators, 16 addresses), i.e. two
+// waves per SIMD, and spends its time waiting: half as many frames per thread and twice
+// the waves keep as many loads in flight and overlap them with the arithmetic.
+constexpr int kHalfFrames = kTileFrames / 2;
+
 template <int VEC, int ACT, class G, int SL>
 __global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
     const void *__restrict__ grad_out, const float *__restrict__ enc,
@@ -255,12 +266,15 @@ __global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
     int t_stride, int u_stride, int D, float *__restrict__ grad_enc,
     float *__restrict__ dec_partial) {
+  static_assert(2 * SL <= kWave, "both halves of a position in one wave");
+  constexpr int kPhases = kBlock / (2 * SL);
   __shared__ __attribute__((aligned(16))) float s_enc[kTileFrames][SL * VEC];
   __shared__ __attribute__((aligned(16))) float s_red[kWavesPerBlock][kTileFrames][SL * VEC];
   const int b = blockIdx.z;
   const int t0 = blockIdx.y * kTileFrames;
   const int lane = threadIdx.x & (SL - 1);
-  const int phase = threadIdx.x / SL;
+  const int half = (threadIdx.x / SL) & 1;
+  const int phase = threadIdx.x / (2 * SL);
   const int col = (blockIdx.x * SL + lane) * VEC;
   const bool col_ok = col < D;  // D is a multiple of VEC
   const int T = min(logit_lengths[b], t_stride);
@@ -272,7 +286,7 @@ __global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
   // output) gets zeros
   const int nframes = max(0, min(kTileFrames, T - t0));
   if (ACT != OT_ACT_NONE) {
-    for (int i = phase; i < kTileFrames; i += (kBlock / SL)) {
+    for (int i = threadIdx.x / SL; i < kTileFrames; i += (kBlock / SL)) {
       Vec<VEC> e;
 #pragma unroll
       for (int k = 0; k < VEC; ++k) e.v[k] = 0.f;
@@ -282,67 +296,71 @@ __global__ __launch_bounds__(kBlock) void joiner_unpack_grad_kernel(
     __syncthreads();
   }
 
-  Vec<VEC> acc[kTileFrames];
+  Vec<VEC> acc[kHalfFrames];
 #pragma unroll
-  for (int i = 0; i < kTileFrames; ++i)
+  for (int i = 0; i < kHalfFrames; ++i)
 #pragma unroll
     for (int k = 0; k < VEC; ++k) acc[i].v[k] = 0.f;
 
   if (nframes > 0 && col_ok) {
     const int64_t frame_stride = (int64_t)U1 * D;
-    for (int u = phase; u < U1; u += (kBlock / SL)) {
+    const int f0 = half * kHalfFrames;  // this thread's first frame of the tile
+    for (int u = phase; u < U1; u += kPhases) {
       const int64_t p = (row0 + (int64_t)t0 * U1 + u) * D + col;
       // frames past the tile's last one re-read frame 0 and are zeroed afterwards: no
       // branch between the loads
-      typename GradIO<G, VEC>::raw_t raw[kTileFrames];
+      typename GradIO<G, VEC>::raw_t raw[kHalfFrames];
 #pragma unroll
-      for (int i = 0; i < kTileFrames; ++i)
-        raw[i] = GradIO<G, VEC>::load(grad_out, p + (i < nframes ? i : 0) * frame_stride);
-      Vec<VEC> g[kTileFrames];
-#pragma unroll
-      for (int i = 0; i < kTileFrames; ++i) {
-        GradIO<G, VEC>::widen(raw[i], g[i]);
-        if (i >= nframes) {
-#pragma unroll
-          for (int k = 0; k < VEC; ++k) g[i].v[k] = 0.f;
-        }
-      }
+      for (int i = 0; i < kHalfFrames; ++i)
+        raw[i] = GradIO<G, VEC>::load(grad_out, p + (f0 + i < nframes ? f0 + i : 0) * frame_stride);
       Vec<VEC> d, sum;
 #pragma unroll
       for (int k = 0; k < VEC; ++k) sum.v[k] = 0.f;
       if (ACT != OT_ACT_NONE) d.load_cached(dec + ((int64_t)(b * u_stride + u) * D + col));
 #pragma unroll
-      for (int i = 0; i < kTileFrames; ++i) {
+      for (int i = 0; i < kHalfFrames; ++i) {
+        Vec<VEC> g;
+        GradIO<G, VEC>::widen(raw[i], g);
+        if (f0 + i >= nframes) {
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) g.v[k] = 0.f;
+        }
         if (ACT != OT_ACT_NONE) {
           Vec<VEC> e;
-          e.load_lds(&s_enc[i][lane * VEC]);
+          e.load_lds(&s_enc[f0 + i][lane * VEC]);
 #pragma unroll
-          for (int k = 0; k < VEC; ++k) g[i].v[k] *= activate_slope<ACT>(e.v[k] + d.v[k]);
+          for (int k = 0; k < VEC; ++k) g.v[k] *= activate_slope<ACT>(e.v[k] + d.v[k]);
         }
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
-          sum.v[k] += g[i].v[k];
-          acc[i].v[k] += g[i].v[k];
+          sum.v[k] += g.v[k];
+          acc[i].v[k] += g.v[k];
         }
       }
-      sum.store(dec_partial + ((((int64_t)b * ntiles + blockIdx.y) * u_stride + u) * D + col));
+      // frames 0-7 + frames 8-15, in that order in both lanes: the same bits as one sum
+      // over the halves' sums on every run
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        const float other = __shfl_xor(sum.v[k], SL, kWave);
+        sum.v[k] = half == 0 ? sum.v[k] + other : other + sum.v[k];
+      }
+      if (half == 0)
+        sum.store(dec_partial + ((((int64_t)b * ntiles + blockIdx.y) * u_stride + u) * D + col));
     }
   }
 
-  // encoder: add the 4 phases of a wave (lanes l, l+16, l+32, l+48), then the waves
+  // encoder: add the phases of a wave (lanes 2 * SL apart), then the waves
+  if (2 * SL < kWave) {
 #pragma unroll
-  for (int i = 0; i < kTileFrames; ++i)
+    for (int i = 0; i < kHalfFrames; ++i)
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) {
-      float v = acc[i].v[k];
-      if (SL <= 16) v += __shfl_xor(v, 16, kWave);
-      if (SL <= 32) v += __shfl_xor(v, 32, kWave);
-      acc[i].v[k] = v;
-    }
+      for (int k = 0; k < VEC; ++k) acc[i].v[k] += __shfl_xor(acc[i].v[k], 2 * SL, kWave);
+  }
   const int wave = threadIdx.x / kWave;
-  if ((threadIdx.x & (kWave - 1)) < SL) {
+  if ((threadIdx.x & (kWave - 1)) < 2 * SL) {
 #pragma unroll
-    for (int i = 0; i < kTileFrames; ++i) acc[i].store_lds(&s_red[wave][i][lane * VEC]);
+    for (int i = 0; i < kHalfFrames; ++i)
+      acc[i].store_lds(&s_red[wave][half * kHalfFrames + i][lane * VEC]);
   }
   __syncthreads();
   // 16 frames x SL (frame, lane) pairs over the workgroup's threads
