@@ -145,26 +145,51 @@ __device__ __forceinline__ int find_utterance(const int32_t *splits, int n, int6
   return lo;
 }
 
+// find_utterance by a whole wave: every lane returns the number of b in [1, n-1] with
+// splits[b] <= row, which is that b (splits ascending, splits[0] = 0 <= row).
+__device__ __forceinline__ int find_utterance_wave(const int32_t *__restrict__ splits, int n,
+                                                   int64_t row) {
+  const int lane = threadIdx.x & (kWave - 1);
+  int count = 0;
+  for (int base = 1; base < n; base += kWave) {
+    const int i = base + lane;
+    const bool le = i < n && (int64_t)splits[i] <= row;
+    count += __builtin_popcountll(__ballot(le));
+  }
+  return count;
+}
+
 // Utterance table of one workgroup of a per-row streaming kernel.  A workgroup
 // owns a contiguous span of at most kMaxRowsPerBlock rows, which can touch at
 // most that many + 1 utterances (every utterance has at least one row), so the
 // slice of row_splits it needs always fits this fixed LDS footprint.
 struct BlockUtterances {
   int32_t splits[kMaxRowsPerBlock + 2];
-  int32_t b_lo;
-  int32_t count;  // utterances touched
+  int32_t b_lo, b_hi;  // utterances of the block's first and last row
+  // utterances touched
+  __device__ __forceinline__ int count() const { return min(b_hi - b_lo + 1, kMaxRowsPerBlock + 1); }
 
-  // Collective over the workgroup; row_first <= row_last are the block's rows.
+  // Collective over the workgroup (at least one whole wave); row_first <= row_last are
+  // the block's rows.  The two searches run in two waves at once (in wave 0 one after
+  // the other for a one-wave workgroup), each as one round of 64 parallel comparisons per
+  // 64 utterances instead of a chain of log2(N) dependent loads.
   __device__ __forceinline__ void load(const int32_t *__restrict__ row_splits, int N,
                                        int64_t row_first, int64_t row_last) {
-    if (threadIdx.x == 0) {
-      const int lo = find_utterance(row_splits, N, row_first);
-      const int hi = find_utterance(row_splits, N, row_last);
-      b_lo = lo;
-      count = min(hi - lo + 1, kMaxRowsPerBlock + 1);
+    const int wave = threadIdx.x / kWave;
+    const bool two = blockDim.x >= 2 * kWave;
+    if (wave == 0) {
+      const int lo = find_utterance_wave(row_splits, N, row_first);
+      if (threadIdx.x == 0) b_lo = lo;
+      if (!two) {
+        const int hi = find_utterance_wave(row_splits, N, row_last);
+        if (threadIdx.x == 0) b_hi = hi;
+      }
+    } else if (wave == 1) {
+      const int hi = find_utterance_wave(row_splits, N, row_last);
+      if (threadIdx.x == kWave) b_hi = hi;
     }
     __syncthreads();
-    const int n = count + 1;
+    const int n = count() + 1;
     for (int i = threadIdx.x; i < n && i < kMaxRowsPerBlock + 2; i += blockDim.x)
       splits[i] = row_splits[b_lo + i];
     __syncthreads();
@@ -172,7 +197,7 @@ struct BlockUtterances {
 
   // Utterance of a row inside the block's span.
   __device__ __forceinline__ int utterance_of(int64_t row) const {
-    return b_lo + find_utterance(splits, count, row);
+    return b_lo + find_utterance(splits, count(), row);
   }
   __device__ __forceinline__ int32_t split(int b) const { return splits[b - b_lo]; }
 };
