@@ -35,7 +35,7 @@ def log_softmax32(x):
 
 # Roundings of size ulp(|log-likelihood|) that two float32 evaluations of one gradient
 # entry may differ by (see lattice_noise_tolerance).
-NOISE_K = 8.0
+NOISE_K = 4.0
 
 
 def lattice_noise_tolerance(ref_grad, loss_per_row, mag, k=NOISE_K, scale=1.0):
