@@ -6,10 +6,9 @@ on ``sys.path`` (or install it) and the import line of existing code need not
 change.  Importing fails, like ``optimized_transducer_amd`` itself, when the HIP
 extension has not been built.
 """
-import optimized_transducer_amd  # noqa: F401  (fails here when the HIP extension is not built)
-
 # through the submodule, as the reference does, so that the function and not the
-# submodule ends up under the name `transducer_loss`
+# submodule ends up under the name `transducer_loss` (fails here when the HIP extension
+# is not built)
 from .transducer_loss import TransducerLoss, TransducerLossFunction, transducer_loss  # noqa: F401,E402
 
 __all__ = ["TransducerLoss", "transducer_loss"]

@@ -18,7 +18,11 @@ def _ensure_built():
     pkg = os.path.join(ROOT, "optimized_transducer_amd")
     if not (os.path.exists(os.path.join(pkg, "libot_transducer.so"))
             and os.path.exists(os.path.join(pkg, "_optimized_transducer.so"))):
-        from optimized_transducer_amd import build
+        # the build script by path, so that the package is first imported once its extension exists
+        import importlib.util
+        spec = importlib.util.spec_from_file_location("_ot_build", os.path.join(pkg, "build.py"))
+        build = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(build)
         build.build_all()
     from oracle import oracle
     oracle.build()
