@@ -501,7 +501,8 @@ def main():
     per_step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(K))
 
     out = {
-        "metric": "utterances/sec fwd+bwd loss at N=32,V=500 fp32; achieved HBM GB/s vs peak",
+        # the headline metric's name on the headline workload (N=32, V=500)
+        "metric": "utterances/sec fwd+bwd loss at N=%d,V=%d fp32; achieved HBM GB/s vs peak" % (w.N, w.V),
         "value": w.N * K / elapsed, "unit": "utterances/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": 1e3 * elapsed / K, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None,
