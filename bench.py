@@ -326,8 +326,19 @@ def bench_project(args):
     T = torch.from_numpy(w.logit_lengths).to(dev)
     U = torch.from_numpy(w.target_lengths).to(dev)
 
+    # --vocab-multiple m: the fused variant runs on a vocabulary padded with masked entries
+    # to the next multiple of m (same loss, same gradient in the real columns), as
+    # project_joiner(..., vocab_multiple=m) does; the weight is padded once, outside the step
+    wt_f, bias_f = wt, bias
+    if args.vocab_multiple and V % args.vocab_multiple:
+        Vp = -(-V // args.vocab_multiple) * args.vocab_multiple
+        wt_f = torch.zeros((Vp, D), dtype=act, device=dev)
+        wt_f[:V] = wt
+        bias_f = torch.full((Vp,), float("-inf"), device=dev)
+        bias_f[:V] = bias
+
     def fused():
-        logits, den = ext.joiner_project(x=x, weight=wt, bias=bias, float32_logits=f32_logits)
+        logits, den = ext.joiner_project(x=x, weight=wt_f, bias=bias_f, float32_logits=f32_logits)
         logits.requires_grad_(True)
         loss = ot.transducer_loss(logits, targets, T, U, w.blank, False, w.one_sym_per_frame,
                                   "sum", denominators=den)
@@ -356,7 +367,7 @@ def bench_project(args):
 
     elapsed = timed(fused)
     elapsed_unfused = timed(unfused)
-    flops = 2.0 * R * D * V
+    flops = 2.0 * R * D * V  # of the real columns, padded or not
     out = {
         "metric": "utterances/sec joiner output projection (fused denominators) + transducer loss "
                   "fwd+bwd; achieved MFMA TFLOP/s of the projection vs peak",
@@ -366,7 +377,8 @@ def bench_project(args):
         "data": "synthetic",
         "config": {"workload": "joiner_projection_of_" + w.name, "N": N, "D": D, "V": V,
                    "packed_rows": R, "activations": str(act).split(".")[-1],
-                   "logits": "f32" if f32_logits else str(act).split(".")[-1]},
+                   "logits": "f32" if f32_logits else str(act).split(".")[-1],
+                   "fused_vocabulary_columns": int(wt_f.shape[0])},
         "unfused": {"ms_per_step": 1e3 * elapsed_unfused / K,
                     "what": "torch (hipBLASLt) projection of the same operands, then the loss with "
                             "its own denominator pass"},
@@ -415,6 +427,9 @@ def main():
                          "the joiner's output projection fused with the denominators "
                          "(project_joiner), then the loss forward + backward")
     ap.add_argument("--joiner-dim", type=int, default=512)
+    ap.add_argument("--vocab-multiple", type=int, default=0,
+                    help="--op project: pad the fused variant's vocabulary with masked entries to "
+                         "a multiple of this (32: whole 128-byte lines per float32 row)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--no-parity", action="store_true",

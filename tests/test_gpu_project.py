@@ -133,6 +133,52 @@ def test_python_pipeline_matches_the_unfused_one(dtype, f32_logits, device):
             (np.abs(a - b_).max(), scale)
 
 
+@pytest.mark.parametrize("f32_logits", [True, False])
+@pytest.mark.parametrize("bias", [True, False])
+def test_padded_vocabulary_changes_nothing_but_the_shape(bias, f32_logits, device):
+    """vocab_multiple: masked entries up to the next multiple.  Same logits and denominators
+    in the real columns, -inf in the others; same loss; the same gradient bits with respect
+    to the logits' real columns, zeros in the others; gradients of x, W, bias as without."""
+    import optimized_transducer_amd as ot
+    dt = torch.bfloat16
+    rng = np.random.default_rng(23)
+    T, U, tg, _ = helpers.random_batch(rng, 5, 11, 6, 8)
+    rows, D, V = int((T * (U + 1)).sum()), 128, 90
+    tg = (tg % (V - 1) + 1).astype(np.int32)
+    x0, w0, b0 = _inputs(rng, rows, D, V, dt, device)
+    dT, dU, dtg = (torch.from_numpy(a).to(device) for a in (T, U, tg))
+
+    def run(multiple):
+        x, w = x0.clone().requires_grad_(True), w0.clone().requires_grad_(True)
+        b = b0.clone().requires_grad_(True) if bias else None
+        logits, den = ot.project_joiner(x, w, b, float32_logits=f32_logits, vocab_multiple=multiple)
+        leaf = logits.detach().clone().requires_grad_(True)
+        loss = ot.transducer_loss(leaf, dtg, dT, dU, 0, False, reduction="sum", denominators=den)
+        loss.backward()
+        logits.backward(leaf.grad)
+        return (logits.detach().clone(), den.clone(), loss.detach(), leaf.grad, x.grad, w.grad,
+                b.grad if bias else None)
+
+    plain = run(None)
+    padded = run(32)
+    assert plain[0].shape == (rows, V) and padded[0].shape == (rows, 96)
+    assert torch.equal(padded[0][:, :V], plain[0]) and torch.isneginf(padded[0][:, V:]).all()
+    assert torch.equal(padded[1], plain[1]) and torch.equal(padded[2], plain[2])
+    assert torch.equal(padded[3][:, :V], plain[3]) and (padded[3][:, V:] == 0).all()
+    # the backward products see V_p instead of V columns: the library may sum in another order
+    for a, b_ in zip(padded[4:], plain[4:]):
+        if b_ is None:
+            assert a is None
+            continue
+        assert a.shape == b_.shape
+        scale = b_.float().abs().max().item()
+        assert (a.float() - b_.float()).abs().max().item() <= 0.02 * scale + 1e-6
+    # a multiple that V already is: nothing is padded
+    assert ot.project_joiner(x0, w0[:64].contiguous(), None, vocab_multiple=32)[0].shape == (rows, 64)
+    with pytest.raises(ValueError, match="vocab_multiple"):
+        ot.project_joiner(x0, w0, b0, vocab_multiple=0)
+
+
 def test_denominators_argument_is_checked(device):
     import optimized_transducer_amd as ot
     rng = np.random.default_rng(2)
