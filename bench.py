@@ -213,6 +213,26 @@ def parity_record(w, args, pristine, targets, T, U, ref, with_f64):
     return rec
 
 
+def timed_steps(torch, step, K, W):
+    """W untimed steps, then K timed ones between two synchronisations; also the spread
+    of the K steps, each between two events on the launch stream.  Returns (seconds,
+    {"median", "min", "max"} in milliseconds)."""
+    for _ in range(W):
+        step()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(K + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    marks[0].record()
+    for i in range(K):
+        step()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(K))
+    median = ms[K // 2] if K % 2 else 0.5 * (ms[K // 2 - 1] + ms[K // 2])
+    return elapsed, {"median": median, "min": ms[0], "max": ms[-1]}
+
+
 def bench_joiner(args):
     """Secondary benchmark: the packed joiner input (pack_joiner, tanh) forward +
     backward for the lengths of the chosen workload; not the headline metric."""
@@ -242,19 +262,12 @@ def bench_joiner(args):
         x = ot.pack_joiner(enc, dec, T, U, activation="tanh", out_dtype=out_dtype)
         x.backward(g)
 
-    for _ in range(W):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(K):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    elapsed, spread = timed_steps(torch, step, K, W)
     out = {
         "metric": "utterances/sec packed joiner input (tanh) fwd+bwd; achieved HBM GB/s vs peak",
         "value": N * K / elapsed, "unit": "utterances/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": 1e3 * elapsed / K, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32" if esize == 4 else "f32->" + args.logits_dtype,
+        "vs_baseline": None, "step_ms": spread, "dtype": "f32" if esize == 4 else "f32->" + args.logits_dtype,
         "data": "synthetic",
         "config": {"workload": "joiner_input_of_" + w.name, "N": N, "D": D, "packed_rows": R,
                    "T_max": Tm, "U1_max": U1m, "activation": "tanh", "packed_bytes": esize * R * D},
@@ -355,31 +368,22 @@ def bench_project(args):
         loss = ot.transducer_loss(logits, targets, T, U, w.blank, False, w.one_sym_per_frame, "sum")
         loss.backward()
 
-    def timed(step):
-        for _ in range(W):
-            step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(K):
-            step()
-        torch.cuda.synchronize()
-        return time.perf_counter() - t0
-
-    elapsed = timed(fused)
-    elapsed_unfused = timed(unfused)
+    elapsed, spread = timed_steps(torch, fused, K, W)
+    elapsed_unfused, spread_unfused = timed_steps(torch, unfused, K, W)
     flops = 2.0 * R * D * V  # of the real columns, padded or not
     out = {
         "metric": "utterances/sec joiner output projection (fused denominators) + transducer loss "
                   "fwd+bwd; achieved MFMA TFLOP/s of the projection vs peak",
         "value": N * K / elapsed, "unit": "utterances/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": 1e3 * elapsed / K, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": args.logits_dtype if not f32_logits else "bf16->f32",
+        "vs_baseline": None, "step_ms": spread,
+        "dtype": args.logits_dtype if not f32_logits else "bf16->f32",
         "data": "synthetic",
         "config": {"workload": "joiner_projection_of_" + w.name, "N": N, "D": D, "V": V,
                    "packed_rows": R, "activations": str(act).split(".")[-1],
                    "logits": "f32" if f32_logits else str(act).split(".")[-1],
                    "fused_vocabulary_columns": int(wt_f.shape[0])},
-        "unfused": {"ms_per_step": 1e3 * elapsed_unfused / K,
+        "unfused": {"ms_per_step": 1e3 * elapsed_unfused / K, "step_ms": spread_unfused,
                     "what": "torch (hipBLASLt) projection of the same operands, then the loss with "
                             "its own denominator pass"},
     }
