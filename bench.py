@@ -183,6 +183,26 @@ def parity_record(w, args, pristine, targets, T, U, ref, with_f64):
         "scores_allclose_rtol1e-5_atol1e-5": bool(torch.allclose(got_scores, ref["scores"], rtol=1e-5, atol=1e-5)),
     }
     del diff, big, within
+    # the integer part of the gate, through the C ABI: row offsets and the row -> utterance
+    # map against numpy's cumsum / repeat, bit for bit
+    import ctypes
+    lib = ctypes.CDLL(os.path.join(ROOT, "optimized_transducer_amd", "libot_transducer.so"))
+    N = int(T.numel())
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    splits = torch.empty(N + 1, dtype=torch.int32, device=T.device)
+    status = torch.zeros(64, dtype=torch.uint8, device=T.device)
+    ids = torch.empty(w.rows, dtype=torch.int32, device=T.device)
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    rc = lib.ot_row_splits(ptr(T), ptr(U), ptr(targets), ctypes.c_int32(N),
+                           ctypes.c_int32(int(targets.shape[1])), ptr(splits), ctypes.c_void_p(None),
+                           ptr(status), stream)
+    rc = rc or lib.ot_row_ids(ptr(splits), ctypes.c_int32(N), ctypes.c_int64(w.rows), ptr(ids), stream)
+    sizes = w.logit_lengths.astype(np.int64) * (w.target_lengths.astype(np.int64) + 1)
+    want_splits = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    rec["row_splits_bit_equal"] = bool(rc == 0 and np.array_equal(splits.cpu().numpy(), want_splits))
+    rec["row_ids_bit_equal"] = bool(rc == 0 and np.array_equal(
+        ids.cpu().numpy(), np.repeat(np.arange(N, dtype=np.int32), sizes)))
+    del splits, status, ids
     if with_f64:
         # the same recursions in float64 as the arbiter between two float32 evaluations
         x = pristine.float().cpu().numpy()
