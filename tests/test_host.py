@@ -34,6 +34,32 @@ def test_library_exports_every_symbol_the_header_declares():
         assert hasattr(lib, n), n
 
 
+def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
+    # the boundary is a C ABI: a C99 translation unit that includes the header and calls an
+    # entry point which needs no device must compile with gcc, link and run
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_abi.c"
+    src.write_text(
+        '#include <stdio.h>\n#include "ot_transducer.h"\n'
+        "int main(void) {\n"
+        "  ot_batch_status s; (void)s;\n"
+        "  if (sizeof(ot_batch_status) != 32) return 2;\n"
+        "  if (ot_workspace_bytes(0, 10) != 0) return 3;\n"
+        "  if (ot_transducer_loss_static(0, 0, 0, 0, 0, 1, 0, 1, 4, 0, 0, 0, 1.0f, 0, 0, 0, 0) >= 0) return 4;\n"
+        '  printf("%s\\n", ot_error_string(OT_E_TOO_LARGE));\n'
+        "  return 0;\n}\n")
+    exe = tmp_path / "use_abi"
+    libdir = os.path.dirname(cabi.LIB_PATH)
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I",
+                    os.path.dirname(cabi.HEADER), str(src), "-o", str(exe), "-L", libdir,
+                    "-l:" + os.path.basename(cabi.LIB_PATH), "-Wl,-rpath," + libdir], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    assert "OT_STATIC_WORKSPACE_BYTES" in out or "static" in out.lower(), out
+
+
 def test_c_abi_rejects_bad_arguments_before_touching_the_device():
     L = cabi.lib()
     null = ctypes.c_void_p(0)
