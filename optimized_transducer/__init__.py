@@ -10,5 +10,8 @@ extension has not been built.
 # submodule ends up under the name `transducer_loss` (fails here when the HIP extension
 # is not built)
 from .transducer_loss import TransducerLoss, TransducerLossFunction, transducer_loss  # noqa: F401,E402
+# what this build has beyond the reference, under the same roof
+from optimized_transducer_amd import joiner_transducer_loss, pack_joiner, project_joiner  # noqa: F401,E402
 
-__all__ = ["TransducerLoss", "transducer_loss"]
+__all__ = ["TransducerLoss", "transducer_loss", "pack_joiner", "project_joiner",
+           "joiner_transducer_loss"]

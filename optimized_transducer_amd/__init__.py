@@ -25,8 +25,8 @@ if _load_error is None:
         )
 
     from .transducer_loss import TransducerLoss, TransducerLossFunction, transducer_loss  # noqa: E402,F401
-    from .joiner import (PackJoinerFunction, ProjectJoinerFunction, pack_joiner,  # noqa: E402,F401
-                         project_joiner)
+    from .joiner import (PackJoinerFunction, ProjectJoinerFunction, joiner_transducer_loss,  # noqa: E402,F401
+                         pack_joiner, project_joiner)
 else:
     # Nothing works without the extension, and nothing pretends to: every name of the
     # package raises.  The import of the bare package itself succeeds so that
@@ -38,4 +38,4 @@ else:
         ) from _load_error
 
 __all__ = ["TransducerLoss", "TransducerLossFunction", "transducer_loss", "PackJoinerFunction",
-           "pack_joiner", "ProjectJoinerFunction", "project_joiner"]
+           "pack_joiner", "ProjectJoinerFunction", "project_joiner", "joiner_transducer_loss"]

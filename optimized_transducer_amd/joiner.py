@@ -165,3 +165,31 @@ def project_joiner(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
         raise ValueError("project_joiner: vocab_multiple must be a positive integer or None, "
                          "got %r" % (vocab_multiple,))
     return ProjectJoinerFunction.apply(x, weight, bias, float32_logits, vocab_multiple)
+
+
+def joiner_transducer_loss(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                           targets: torch.Tensor, logit_lengths: torch.Tensor,
+                           target_lengths: torch.Tensor, blank: int,
+                           one_sym_per_frame: bool = False, reduction: str = "mean",
+                           float32_logits: bool = True) -> torch.Tensor:
+    """``transducer_loss(linear(x), ...)`` for a joiner under mixed precision, in the
+    fastest arrangement this package has: the projection on the matrix cores with
+    the loss's denominators as a by-product (:func:`project_joiner`), the vocabulary
+    padded to a multiple of 32 with masked entries so that every row of logits is a
+    whole number of cache lines, and the loss started from its gather step.  The
+    logits never leave this function, so their padded shape concerns nobody.
+
+    Args:
+      x, weight, bias, float32_logits: as for :func:`project_joiner`.
+      targets, logit_lengths, target_lengths, blank, one_sym_per_frame, reduction:
+        as for :func:`transducer_loss` (README.md:179-187 of the reference).
+    Returns:
+      The loss, differentiable in ``x``, ``weight`` and ``bias``; the same number,
+      and the same gradients, as ``transducer_loss(project_joiner(x, weight,
+      bias)[0], ..., from_log_softmax=False)``.
+    """
+    from .transducer_loss import transducer_loss
+    logits, den = project_joiner(x, weight, bias, float32_logits=float32_logits, vocab_multiple=32)
+    return transducer_loss(logits, targets, logit_lengths, target_lengths, blank, False,
+                           one_sym_per_frame, reduction, denominators=den)
+

@@ -179,6 +179,34 @@ def test_padded_vocabulary_changes_nothing_but_the_shape(bias, f32_logits, devic
         ot.project_joiner(x0, w0, b0, vocab_multiple=0)
 
 
+@pytest.mark.parametrize("osf", [False, True])
+def test_joiner_transducer_loss_is_the_two_calls_in_one(osf, device):
+    import optimized_transducer_amd as ot
+    dt = torch.bfloat16
+    rng = np.random.default_rng(29)
+    T, U, tg, _ = helpers.random_batch(rng, 4, 10, 5, 8, one_sym_per_frame=osf)
+    rows, D, V = int((T * (U + 1)).sum()), 64, 45
+    tg = (tg % (V - 1) + 1).astype(np.int32)
+    x0, w0, b0 = _inputs(rng, rows, D, V, dt, device)
+    dT, dU, dtg = (torch.from_numpy(a).to(device) for a in (T, U, tg))
+
+    def run(one_call):
+        x, w, b = (t.clone().requires_grad_(True) for t in (x0, w0, b0))
+        if one_call:
+            loss = ot.joiner_transducer_loss(x, w, b, dtg, dT, dU, 0, osf, "sum")
+        else:
+            logits, den = ot.project_joiner(x, w, b)
+            loss = ot.transducer_loss(logits, dtg, dT, dU, 0, False, osf, "sum", denominators=den)
+        loss.backward()
+        return loss.detach(), x.grad, w.grad, b.grad
+
+    a, b_ = run(True), run(False)
+    assert torch.equal(a[0], b_[0])
+    for p, q in zip(a[1:], b_[1:]):
+        scale = q.float().abs().max().item()
+        assert p.shape == q.shape and (p.float() - q.float()).abs().max().item() <= 0.02 * scale + 1e-6
+
+
 def test_denominators_argument_is_checked(device):
     import optimized_transducer_amd as ot
     rng = np.random.default_rng(2)

@@ -185,6 +185,9 @@ def test_the_reference_import_line_works():
     assert optimized_transducer.TransducerLoss is ot.TransducerLoss
     from optimized_transducer.transducer_loss import TransducerLossFunction
     assert TransducerLossFunction is ot.TransducerLossFunction
+    # the additions are reachable under the same name
+    for name in ("pack_joiner", "project_joiner", "joiner_transducer_loss"):
+        assert getattr(optimized_transducer, name) is getattr(ot, name)
 
 
 def test_reduction_none_is_rejected_like_the_reference():
