@@ -304,6 +304,7 @@ int ot_transducer_loss_static(const float *logits, const int32_t *targets,
  * all float32 and contiguous. */
 #define OT_ACT_NONE 0 /* out = enc + dec                                      */
 #define OT_ACT_TANH 1 /* out = tanh(enc + dec)                                */
+#define OT_ACT_RELU 2 /* out = max(enc + dec, 0)                              */
 #define OT_JOINER_TILE_FRAMES 16 /* frames per partial decoder sum            */
 
 /* out (rows, D), rows = row_splits[N]: for utterance b and cell (t, u),
@@ -324,7 +325,7 @@ int ot_joiner_pack(const float *enc, const float *dec,
  * full.  One pass over grad_out; the decoder sums go through per-16-frame
  * partial sums in `workspace` (16-byte aligned, ot_joiner_unpack_workspace_bytes)
  * and are added in a fixed order, so results do not vary from run to run.
- * enc and dec are read only for OT_ACT_TANH (may be NULL otherwise). */
+ * enc and dec are read only for OT_ACT_TANH and OT_ACT_RELU (may be NULL otherwise). */
 size_t ot_joiner_unpack_workspace_bytes(int32_t N, int32_t t_stride,
                                         int32_t u_stride, int32_t D);
 int ot_joiner_unpack_grad(const float *grad_out, const float *enc,

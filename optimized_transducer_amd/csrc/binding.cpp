@@ -603,7 +603,8 @@ void scale_by_device_scalar_(torch::Tensor &x, const torch::Tensor &factor) {
 int activation_code(const std::string &name) {
   if (name == "none") return OT_ACT_NONE;
   if (name == "tanh") return OT_ACT_TANH;
-  TORCH_CHECK(false, "activation must be 'none' or 'tanh', got '", name, "'");
+  if (name == "relu") return OT_ACT_RELU;
+  TORCH_CHECK(false, "activation must be 'none', 'tanh' or 'relu', got '", name, "'");
   return -1;
 }
 

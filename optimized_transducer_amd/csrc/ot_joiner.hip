@@ -39,7 +39,7 @@ __device__ __forceinline__ float tanh_dev(float x) {
 
 template <int ACT>
 __device__ __forceinline__ float activate(float s) {
-  return ACT == OT_ACT_TANH ? tanh_dev(s) : s;
+  return ACT == OT_ACT_TANH ? tanh_dev(s) : ACT == OT_ACT_RELU ? fmaxf(s, 0.f) : s;
 }
 
 // tanh for a result that is rounded to 8 or 11 significant bits afterwards:
@@ -54,7 +54,7 @@ __device__ __forceinline__ float tanh_16bit(float x) {
 }
 template <int ACT>
 __device__ __forceinline__ float activate_16bit(float s) {
-  return ACT == OT_ACT_TANH ? tanh_16bit(s) : s;
+  return ACT == OT_ACT_TANH ? tanh_16bit(s) : ACT == OT_ACT_RELU ? fmaxf(s, 0.f) : s;
 }
 // d act(s) / d s
 template <int ACT>
@@ -65,6 +65,7 @@ __device__ __forceinline__ float activate_slope(float s) {
     const float r = __builtin_amdgcn_rcpf(1.f + e);
     return 4.f * e * (r * r);
   }
+  if (ACT == OT_ACT_RELU) return s > 0.f ? 1.f : 0.f;  // 0 at s = 0, like torch.relu's backward
   return 1.f;
 }
 
@@ -417,6 +418,9 @@ __global__ __launch_bounds__(kBlock) void joiner_dec_reduce_kernel(
 static inline int launch_status() { return (int)hipGetLastError(); }
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 static inline bool aligned4(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 3) == 0; }
+static inline bool known_activation(int32_t a) {
+  return a == OT_ACT_NONE || a == OT_ACT_TANH || a == OT_ACT_RELU;
+}
 
 }  // namespace ot
 
@@ -431,7 +435,7 @@ int ot_joiner_pack(const float *enc, const float *dec, const int32_t *logit_leng
   if (!enc || !dec || !logit_lengths || !target_lengths || !row_splits || !out || N <= 0 ||
       N > 65535 || t_stride <= 0 || u_stride <= 0 || D <= 0 ||
       (int64_t)N * t_stride > INT32_MAX || (int64_t)N * u_stride > INT32_MAX ||
-      (activation != OT_ACT_NONE && activation != OT_ACT_TANH))
+      !known_activation(activation))
     return OT_E_BAD_ARG;
   if (!aligned4(enc) || !aligned4(dec) || !aligned4(out)) return OT_E_MISALIGNED;
   if ((t_stride + kPackFrames - 1) / kPackFrames > 65535) return OT_E_TOO_LONG;
@@ -446,6 +450,8 @@ int ot_joiner_pack(const float *enc, const float *dec, const int32_t *logit_leng
                      logit_lengths, target_lengths, row_splits, t_stride, u_stride, D, out)
   if (activation == OT_ACT_TANH) {
     if (vec == 4) OT_LAUNCH_PACKT(4, OT_ACT_TANH); else OT_LAUNCH_PACKT(1, OT_ACT_TANH);
+  } else if (activation == OT_ACT_RELU) {
+    if (vec == 4) OT_LAUNCH_PACKT(4, OT_ACT_RELU); else OT_LAUNCH_PACKT(1, OT_ACT_RELU);
   } else {
     if (vec == 4) OT_LAUNCH_PACKT(4, OT_ACT_NONE); else OT_LAUNCH_PACKT(1, OT_ACT_NONE);
   }
@@ -460,7 +466,7 @@ int ot_joiner_pack_half(const float *enc, const float *dec, const int32_t *logit
   if (!enc || !dec || !logit_lengths || !target_lengths || !row_splits || !out || N <= 0 ||
       N > 65535 || t_stride <= 0 || u_stride <= 0 || D <= 0 || D % 8 != 0 ||
       (int64_t)N * t_stride > INT32_MAX || (int64_t)N * u_stride > INT32_MAX ||
-      (activation != OT_ACT_NONE && activation != OT_ACT_TANH) ||
+      !known_activation(activation) ||
       (out_dtype != OT_DTYPE_F16 && out_dtype != OT_DTYPE_BF16))
     return OT_E_BAD_ARG;
   if (!aligned16(enc) || !aligned16(dec) || !aligned16(out)) return OT_E_MISALIGNED;
@@ -476,6 +482,8 @@ int ot_joiner_pack_half(const float *enc, const float *dec, const int32_t *logit
                      logit_lengths, target_lengths, row_splits, t_stride, u_stride, D, o)
   if (activation == OT_ACT_TANH) {
     if (out_dtype == OT_DTYPE_F16) OT_LAUNCH_PACKH(OT_ACT_TANH, F16); else OT_LAUNCH_PACKH(OT_ACT_TANH, BF16);
+  } else if (activation == OT_ACT_RELU) {
+    if (out_dtype == OT_DTYPE_F16) OT_LAUNCH_PACKH(OT_ACT_RELU, F16); else OT_LAUNCH_PACKH(OT_ACT_RELU, BF16);
   } else {
     if (out_dtype == OT_DTYPE_F16) OT_LAUNCH_PACKH(OT_ACT_NONE, F16); else OT_LAUNCH_PACKH(OT_ACT_NONE, BF16);
   }
@@ -501,7 +509,7 @@ int ot_joiner_unpack_grad_from(const void *grad_out, int32_t grad_dtype, const f
   if (!grad_out || !logit_lengths || !target_lengths || !row_splits || !workspace || !grad_enc ||
       !grad_dec || N <= 0 || N > 65535 || t_stride <= 0 || u_stride <= 0 || D <= 0 ||
       (int64_t)N * t_stride > INT32_MAX || (int64_t)N * u_stride > INT32_MAX ||
-      (activation != OT_ACT_NONE && activation != OT_ACT_TANH) ||
+      !known_activation(activation) ||
       (activation != OT_ACT_NONE && (!enc || !dec)))
     return OT_E_BAD_ARG;
   if (workspace_bytes < ot_joiner_unpack_workspace_bytes(N, t_stride, u_stride, D))
@@ -530,6 +538,8 @@ int ot_joiner_unpack_grad_from(const void *grad_out, int32_t grad_dtype, const f
   else OT_LAUNCH_UNPACK(VEC_, ACT_, BF16, kSlabLanesHalf)
   if (activation == OT_ACT_TANH) {
     if (vec == 4) { OT_LAUNCH_UNPACK_G(4, OT_ACT_TANH); } else { OT_LAUNCH_UNPACK_G(1, OT_ACT_TANH); }
+  } else if (activation == OT_ACT_RELU) {
+    if (vec == 4) { OT_LAUNCH_UNPACK_G(4, OT_ACT_RELU); } else { OT_LAUNCH_UNPACK_G(1, OT_ACT_RELU); }
   } else {
     if (vec == 4) { OT_LAUNCH_UNPACK_G(4, OT_ACT_NONE); } else { OT_LAUNCH_UNPACK_G(1, OT_ACT_NONE); }
   }

@@ -74,7 +74,8 @@ def pack_joiner(
         padding.
       logit_lengths: (N,) int32, T_i (1 <= T_i <= T).
       target_lengths: (N,) int32, U_i (0 <= U_i <= U).
-      activation: None / "none" for ``enc + dec``, "tanh" for ``tanh(enc + dec)``.
+      activation: None / "none" for ``enc + dec``, "tanh" for ``tanh(enc + dec)`` (the
+        reference's recipe), "relu" for ``relu(enc + dec)``.
       out_dtype: torch.float32, or torch.float16 / torch.bfloat16 (D a multiple of 8)
         for a projection in 16 bits (:func:`project_joiner`): computed in float32 and
         rounded once, without a float32 array and a cast pass in between.

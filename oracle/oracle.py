@@ -195,7 +195,8 @@ def pack_joiner(encoder_out, decoder_out, logit_lengths, target_lengths, activat
                 dtype=np.float32):
     """The reference's recipe for the joiner input (README.md:166-177), literally:
     per utterance e[:T, None, :] + d[None, :U+1, :], reshaped to (T*(U+1), D),
-    concatenated; then tanh when activation == "tanh"."""
+    concatenated; then tanh when activation == "tanh" (the README's choice), max(x, 0)
+    when activation == "relu"."""
     enc = np.asarray(encoder_out, dtype=dtype)
     dec = np.asarray(decoder_out, dtype=dtype)
     D = enc.shape[2]
@@ -205,13 +206,15 @@ def pack_joiner(encoder_out, decoder_out, logit_lengths, target_lengths, activat
         d = dec[i, :int(target_lengths[i]) + 1, :]
         parts.append((e[:, None, :] + d[None, :, :]).reshape(-1, D))
     x = np.concatenate(parts)
+    if activation == "relu":
+        return np.maximum(x, 0)
     return np.tanh(x) if activation == "tanh" else x
 
 
 def pack_joiner_backward(grad_out, encoder_out, decoder_out, logit_lengths, target_lengths,
                          activation=None, dtype=np.float64):
     """Gradient of pack_joiner by the chain rule: the incoming gradient of a row,
-    times 1 - tanh^2 for "tanh", is added to its encoder frame and to its decoder
+    times 1 - tanh^2 for "tanh" (times [s > 0] for "relu"), is added to its encoder frame and to its decoder
     position; padding receives zero.  Returns (grad_enc, grad_dec, abs_enc, abs_dec):
     the last two are the same sums over the absolute values of the incoming
     gradient, the scale of the rounding error of a float32 evaluation (of the
@@ -231,6 +234,8 @@ def pack_joiner_backward(grad_out, encoder_out, decoder_out, logit_lengths, targ
         if activation == "tanh":
             a = np.tanh(enc[i, :T, None, :] + dec[i, None, :U1, :])
             gi = gi * (1.0 - a * a)
+        elif activation == "relu":
+            gi = gi * ((enc[i, :T, None, :] + dec[i, None, :U1, :]) > 0)
         ge[i, :T] = gi.sum(1)
         gd[i, :U1] = gi.sum(0)
         r += T * U1

@@ -19,7 +19,7 @@ from oracle import oracle
 
 pytestmark = pytest.mark.gpu
 
-ACT = {None: 0, "tanh": 1}
+ACT = {None: 0, "tanh": 1, "relu": 2}
 
 
 def _dev(a, device):
@@ -49,7 +49,7 @@ CASES = [  # name, N, Tmax, U1max, D, pad_t, pad_u
 ]
 
 
-@pytest.mark.parametrize("activation", [None, "tanh"])
+@pytest.mark.parametrize("activation", [None, "tanh", "relu"])
 @pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
 def test_pack_and_unpack_through_the_c_abi(case, activation, device):
     _, N, Tm, U1m, D, pad_t, pad_u = case
@@ -64,7 +64,7 @@ def test_pack_and_unpack_through_the_c_abi(case, activation, device):
     out = cabi.joiner_pack(denc, ddec, dT, dU, splits, rows, ACT[activation]).cpu().numpy()
     # without activation every entry is one float32 addition: bit exact, which also pins the
     # row -> (utterance, frame, position) arithmetic
-    if activation is None:
+    if activation in (None, "relu"):  # (the larger of that sum and 0 is exact as well)
         assert (out == want).all()
     else:
         assert np.allclose(out, want, rtol=1e-6, atol=1e-6), np.abs(out - want).max()
@@ -101,7 +101,7 @@ def test_tanh_accuracy_over_the_whole_range(device):
     assert (np.sign(out) == np.sign(want)).all() and np.abs(out).max() <= 1.0
 
 
-@pytest.mark.parametrize("activation", [None, "tanh"])
+@pytest.mark.parametrize("activation", [None, "tanh", "relu"])
 def test_python_entry_point_and_autograd(activation, device):
     import optimized_transducer_amd as ot
     rng = np.random.default_rng(3)
@@ -120,6 +120,8 @@ def test_python_entry_point_and_autograd(activation, device):
     y = torch.cat(parts)
     if activation == "tanh":
         y = torch.tanh(y)
+    if activation == "relu":
+        y = torch.relu(y)
     assert torch.allclose(x, y, rtol=1e-6, atol=1e-6)
     g = torch.randn_like(x)
     x.backward(g)
@@ -151,7 +153,7 @@ def test_argument_checks(device):
     with pytest.raises(RuntimeError, match="last dimension"):
         ot.pack_joiner(de, dd[:, :, :4].contiguous(), dT, dU)
     with pytest.raises(RuntimeError, match="activation"):
-        ot.pack_joiner(de, dd, dT, dU, activation="relu")
+        ot.pack_joiner(de, dd, dT, dU, activation="gelu")
     with pytest.raises(RuntimeError, match="no CPU"):
         ot.pack_joiner(torch.from_numpy(enc), torch.from_numpy(dec), torch.from_numpy(T),
                        torch.from_numpy(U))
@@ -166,7 +168,7 @@ HALF_CASES = [c for c in CASES if c[4] % 8 == 0]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
-@pytest.mark.parametrize("activation", [None, "tanh"])
+@pytest.mark.parametrize("activation", [None, "tanh", "relu"])
 @pytest.mark.parametrize("case", HALF_CASES, ids=[c[0] for c in HALF_CASES])
 def test_pack_with_16_bit_output(case, activation, dtype, device):
     """float32 arithmetic, one rounding to nearest even: without activation the float32
@@ -181,7 +183,7 @@ def test_pack_with_16_bit_output(case, activation, dtype, device):
     got = cabi.joiner_pack_half(denc, ddec, dT, dU, splits, rows, ACT[activation], dtype)
     full = cabi.joiner_pack(denc, ddec, dT, dU, splits, rows, ACT[activation])
     assert got.dtype == dtype
-    if activation is None:
+    if activation in (None, "relu"):
         assert torch.equal(got, full.to(dtype))
     else:
         one = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7   # one unit in the last place
@@ -230,7 +232,7 @@ def test_pack_16_bit_output_in_the_python_pipeline(device):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
-@pytest.mark.parametrize("activation", [None, "tanh"])
+@pytest.mark.parametrize("activation", [None, "tanh", "relu"])
 @pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
 def test_unpack_of_a_16_bit_gradient(case, activation, dtype, device):
     """The incoming gradient is widened (exactly) inside the kernel, for 4 columns per thread and

@@ -356,7 +356,7 @@ def test_oracle_against_compiled_reference_live(fls, one_sym):
 
 
 # ------------------------------------------------------------ packed joiner input
-def _readme_joiner(encoder_out, decoder_out, logit_lengths, target_lengths, tanh):
+def _readme_joiner(encoder_out, decoder_out, logit_lengths, target_lengths, activation):
     # the reference's usage recipe, README.md:166-177, in torch (float64, autograd)
     N, D = encoder_out.shape[0], encoder_out.shape[2]
     encoder_out_list = [encoder_out[i, :logit_lengths[i], :] for i in range(N)]
@@ -364,10 +364,12 @@ def _readme_joiner(encoder_out, decoder_out, logit_lengths, target_lengths, tanh
     x = [e.unsqueeze(1) + d.unsqueeze(0) for e, d in zip(encoder_out_list, decoder_out_list)]
     x = [p.reshape(-1, D) for p in x]
     x = torch.cat(x)
-    return torch.tanh(x) if tanh else x
+    if activation == "relu":  # not in the README: another activation a joiner may use
+        return torch.relu(x)
+    return torch.tanh(x) if activation == "tanh" else x
 
 
-@pytest.mark.parametrize("activation", [None, "tanh"])
+@pytest.mark.parametrize("activation", [None, "tanh", "relu"])
 def test_pack_joiner_oracle_matches_the_readme_recipe_and_its_autograd(activation):
     rng = np.random.default_rng(11)
     N, Tm, Um, D = 5, 9, 6, 7
@@ -379,7 +381,7 @@ def test_pack_joiner_oracle_matches_the_readme_recipe_and_its_autograd(activatio
     dec = rng.standard_normal((N, Um, D))
     te = torch.tensor(enc, requires_grad=True)
     td = torch.tensor(dec, requires_grad=True)
-    want = _readme_joiner(te, td, T.tolist(), U.tolist(), activation == "tanh")
+    want = _readme_joiner(te, td, T.tolist(), U.tolist(), activation)
     got = oracle.pack_joiner(enc, dec, T, U, activation, dtype=np.float64)
     assert got.shape == tuple(want.shape) == (int((T * (U + 1)).sum()), D)
     assert np.allclose(got, want.detach().numpy(), rtol=1e-14, atol=1e-14)
@@ -388,7 +390,7 @@ def test_pack_joiner_oracle_matches_the_readme_recipe_and_its_autograd(activatio
     b, t, u = 1, 3, 2
     row = splits[b] + t * (U[b] + 1) + u
     s = enc[b, t] + dec[b, u]
-    assert np.allclose(got[row], np.tanh(s) if activation == "tanh" else s)
+    assert np.allclose(got[row], {None: s, "tanh": np.tanh(s), "relu": np.maximum(s, 0)}[activation])
     g = rng.standard_normal(got.shape)
     want.backward(torch.tensor(g))
     ge, gd, ae, ad = oracle.pack_joiner_backward(g, enc, dec, T, U, activation)
