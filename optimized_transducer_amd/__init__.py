@@ -31,8 +31,15 @@ else:
     # Nothing works without the extension, and nothing pretends to: every name of the
     # package raises.  The import of the bare package itself succeeds so that
     # `python -m optimized_transducer_amd.build` can run in an unbuilt tree.
+    class ExtensionNotBuilt(ImportError, AttributeError):
+        """ImportError for `from optimized_transducer_amd import x`; also an AttributeError,
+        so that hasattr(), getattr(..., default) and the import system's probes for
+        submodules and dunder names behave as for any missing attribute."""
+
     def __getattr__(name):
-        raise ImportError(
+        if name.startswith("__") and name.endswith("__"):
+            raise AttributeError(name)
+        raise ExtensionNotBuilt(
             "optimized_transducer_amd: the HIP extension is not built or failed to load (%s). "
             "Run `python -m optimized_transducer_amd.build` in the repository root." % (_load_error,)
         ) from _load_error

@@ -22,10 +22,12 @@ EXT_LIB = os.path.join(HERE, "_optimized_transducer.so")
 # -packed-fp32-ops off: scalar float code must not be fused into v_pk_*_f32.
 # No fast-math, no FP contraction: the float expressions keep their written order.
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-ffp-contract=off", "-fno-fast-math", "-Wall",
 ]
+KERNEL_SOURCES = ("ot_kernels.hip", "ot_joiner.hip", "ot_half.hip", "ot_project.hip")
+OBJ_DIR = os.path.join(HERE, "build")  # objects only; ignored by git
 
 
 def _run(cmd):
@@ -33,10 +35,30 @@ def _run(cmd):
     subprocess.run(cmd, check=True)
 
 
-def build_kernels():
-    srcs = [os.path.join(CSRC, f) for f in ("ot_kernels.hip", "ot_joiner.hip", "ot_half.hip", "ot_project.hip")]
-    _run([os.path.join(ROCM, "bin", "hipcc")] + HIPCC_FLAGS +
-         ["-I", INCLUDE, "-I", CSRC] + srcs + ["-o", KERNEL_LIB])
+def _newer(target, sources):
+    if not os.path.exists(target):
+        return False
+    t = os.path.getmtime(target)
+    return all(os.path.getmtime(x) <= t for x in sources)
+
+
+def build_kernels(incremental=False):
+    """One object per source file, compiled side by side, then one shared library.
+    incremental: keep the objects whose source and headers have not changed since."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    headers += [os.path.join(INCLUDE, f) for f in os.listdir(INCLUDE) if f.endswith(".h")]
+    jobs = []
+    for f in KERNEL_SOURCES:
+        src, obj = os.path.join(CSRC, f), os.path.join(OBJ_DIR, f + ".o")
+        if not (incremental and _newer(obj, [src] + headers)):
+            jobs.append([hipcc] + HIPCC_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c", src, "-o", obj])
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        list(pool.map(_run, jobs))
+    objs = [os.path.join(OBJ_DIR, f + ".o") for f in KERNEL_SOURCES]
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", KERNEL_LIB])
     return KERNEL_LIB
 
 
@@ -69,11 +91,13 @@ def build_extension():
     return EXT_LIB
 
 
-def build_all():
-    build_kernels()
-    build_extension()
+def build_all(incremental=False):
+    build_kernels(incremental)
+    if not (incremental and _newer(EXT_LIB, [os.path.join(CSRC, "binding.cpp"),
+                                            os.path.join(INCLUDE, "ot_transducer.h")])):
+        build_extension()
 
 
 if __name__ == "__main__":
-    build_all()
+    build_all(incremental="--incremental" in sys.argv[1:])
     sys.exit(0)

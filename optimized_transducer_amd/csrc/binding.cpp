@@ -106,6 +106,31 @@ struct EventGuard {
   EventGuard &operator=(const EventGuard &) = delete;
 };
 
+// An event recorded behind a kernel that writes into pinned host memory.  Whoever owns
+// that memory must not release it while the kernel may still run: if the call unwinds
+// (an argument check or a launch throws) before the event has been waited for, the
+// destructor waits.  Declare it after the host tensor so that it is destroyed first.
+struct HostWriteGuard {
+  EventGuard event;
+  hipStream_t stream;
+  bool recorded = false, waited = false;
+  explicit HostWriteGuard(hipStream_t s) : stream(s) {}
+  void record() {
+    OT_CHECK_HIP(hipEventRecord(event.ev, stream));
+    recorded = true;
+  }
+  void wait() {
+    OT_CHECK_HIP(hipEventSynchronize(event.ev));
+    waited = true;
+  }
+  ~HostWriteGuard() {
+    if (waited) return;
+    // unwinding: the kernel may have been launched even if the event was not recorded
+    if (recorded) (void)hipEventSynchronize(event.ev);
+    else (void)hipStreamSynchronize(stream);
+  }
+};
+
 // Batches below this many logits elements run on one stream.
 constexpr int64_t kOverlapMinElements = (int64_t)32 << 20;
 
@@ -292,6 +317,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
       torch::TensorOptions().dtype(torch::kUInt8).device(torch::kCPU).pinned_memory(true));
   void *status_dev = nullptr;
   OT_CHECK_HIP(hipHostGetDevicePointer(&status_dev, status_host.data_ptr(), 0));
+  HostWriteGuard status_ready(stream);  // after status_host: destroyed, i.e. waited for, before it
   {
     ScopedTimer timer("prepare", stream);
     OT_CHECK(ot_row_splits(
@@ -299,8 +325,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
         reinterpret_cast<int32_t *>(static_cast<char *>(status_dev) + host_splits_off),
         static_cast<ot_batch_status *>(status_dev), stream));
   }
-  EventGuard status_ready;
-  OT_CHECK_HIP(hipEventRecord(status_ready.ev, stream));
+  status_ready.record();
 
   // Two-part schedule for large batches.  The lattice kernel is a chain of
   // T+U dependent steps on a handful of CUs; run on a second stream, the part of
@@ -353,7 +378,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
                                    one_sym_per_frame, rows, alpha, beta, scores.data_ptr<float>(),
                                    scores_beta, stream));
   }
-  OT_CHECK_HIP(hipEventSynchronize(status_ready.ev));
+  status_ready.wait();
   const ot_batch_status st = *reinterpret_cast<const ot_batch_status *>(status_host.data_ptr());
   const int32_t *splits_host = reinterpret_cast<const int32_t *>(
       static_cast<const char *>(status_host.data_ptr()) + host_splits_off);
@@ -660,15 +685,15 @@ std::pair<torch::Tensor, torch::Tensor> joiner_pack(
       torch::TensorOptions().dtype(torch::kUInt8).device(torch::kCPU).pinned_memory(true));
   void *status_dev = nullptr;
   OT_CHECK_HIP(hipHostGetDevicePointer(&status_dev, status_host.data_ptr(), 0));
+  HostWriteGuard ready(stream);
   {
     ScopedTimer timer("prepare", stream);
     OT_CHECK(ot_row_splits(logit_lengths.data_ptr<int32_t>(), target_lengths.data_ptr<int32_t>(),
                            nullptr, (int32_t)N, 0, row_splits.data_ptr<int32_t>(), nullptr,
                            static_cast<ot_batch_status *>(status_dev), stream));
   }
-  EventGuard ready;
-  OT_CHECK_HIP(hipEventRecord(ready.ev, stream));
-  OT_CHECK_HIP(hipEventSynchronize(ready.ev));  // the output's size is a batch fact
+  ready.record();
+  ready.wait();  // the output's size is a batch fact
   const ot_batch_status st = *reinterpret_cast<const ot_batch_status *>(status_host.data_ptr());
   TORCH_CHECK(st.logit_len_min >= 1 && st.target_len_min >= 0,
               "pack_joiner: expect logit_lengths >= 1 and target_lengths >= 0, but the minima are ",

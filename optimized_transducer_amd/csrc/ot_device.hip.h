@@ -159,6 +159,15 @@ __device__ __forceinline__ int find_utterance_wave(const int32_t *__restrict__ s
   return count;
 }
 
+// The wave-parallel count reads the whole table (n/64 rounds of independent loads), the
+// binary search log2(n) dependent ones: the first is faster for the few hundred
+// utterances of a usual batch, the second for thousands.
+constexpr int kWaveSearchMax = 1024;
+__device__ __forceinline__ int find_utterance_uniform(const int32_t *__restrict__ splits, int n,
+                                                      int64_t row) {
+  return n <= kWaveSearchMax ? find_utterance_wave(splits, n, row) : find_utterance(splits, n, row);
+}
+
 // Utterance table of one workgroup of a per-row streaming kernel.  A workgroup
 // owns a contiguous span of at most kMaxRowsPerBlock rows, which can touch at
 // most that many + 1 utterances (every utterance has at least one row), so the
@@ -172,20 +181,21 @@ struct BlockUtterances {
   // Collective over the workgroup (at least one whole wave); row_first <= row_last are
   // the block's rows.  The two searches run in two waves at once (in wave 0 one after
   // the other for a one-wave workgroup), each as one round of 64 parallel comparisons per
-  // 64 utterances instead of a chain of log2(N) dependent loads.
+  // 64 utterances instead of a chain of log2(N) dependent loads (up to kWaveSearchMax
+  // utterances; a binary search beyond).
   __device__ __forceinline__ void load(const int32_t *__restrict__ row_splits, int N,
                                        int64_t row_first, int64_t row_last) {
     const int wave = threadIdx.x / kWave;
     const bool two = blockDim.x >= 2 * kWave;
     if (wave == 0) {
-      const int lo = find_utterance_wave(row_splits, N, row_first);
+      const int lo = find_utterance_uniform(row_splits, N, row_first);
       if (threadIdx.x == 0) b_lo = lo;
       if (!two) {
-        const int hi = find_utterance_wave(row_splits, N, row_last);
+        const int hi = find_utterance_uniform(row_splits, N, row_last);
         if (threadIdx.x == 0) b_hi = hi;
       }
     } else if (wave == 1) {
-      const int hi = find_utterance_wave(row_splits, N, row_last);
+      const int hi = find_utterance_uniform(row_splits, N, row_last);
       if (threadIdx.x == kWave) b_hi = hi;
     }
     __syncthreads();

@@ -637,13 +637,18 @@ __global__ __launch_bounds__(THREADS) void alpha_beta_staged_kernel(
     const float *__restrict__ lp, const int32_t *__restrict__ logit_lengths,
     const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
     int utt_begin, float *__restrict__ alpha, float *__restrict__ beta,
-    float *__restrict__ scores_alpha, float *__restrict__ scores_beta, int guard_n,
+    float *__restrict__ scores_alpha, float *__restrict__ scores_beta, int max_u1, int guard_n,
     int64_t guard_rows) {
   __shared__ float s_ring[THREADS / kWave][kRing + kChunk];
   extern __shared__ __attribute__((aligned(16))) float s_stage[];
   const int b = utt_begin + blockIdx.x;
   const int T = logit_lengths[b], U = target_lengths[b];
-  if (!lattice_guard_ok(row_splits, guard_n, guard_rows, T, U, (int)blockDim.x)) return;
+  if (!lattice_guard_ok(row_splits, guard_n, guard_rows, T, U, max_u1)) return;
+  // utterances with more columns than this workgroup has threads belong to the tiled launch
+  if (U >= (int)blockDim.x) return;
+  // a wave none of whose lanes has a column takes no part (a barrier only waits for the
+  // waves of the workgroup that have not ended)
+  if ((int)(threadIdx.x / kWave) > U / kWave) return;
   const int64_t row0 = row_splits[b];
   if (blockIdx.y == 0)
     lattice_sweep_staged<false, G>(lp, T, U, row0, alpha, scores_alpha + b, s_ring, s_stage);
@@ -682,6 +687,12 @@ __global__ __launch_bounds__(OT_LATTICE_TILE) void alpha_beta_kernel(
   const int b = utt_begin + blockIdx.x;
   const int T = logit_lengths[b], U = target_lengths[b];
   if (!lattice_guard_ok(row_splits, guard_n, guard_rows, T, U, max_u1)) return;
+  // The tiled launch takes the utterances with more than OT_LATTICE_TILE columns only, the
+  // launch in front of it (same grid) all the others.
+  if (TILED ? U < OT_LATTICE_TILE : U >= (int)blockDim.x) return;
+  // a wave none of whose lanes has a column takes no part (a barrier only waits for the
+  // waves of the workgroup that have not ended)
+  if (MULTI && !TILED && (int)(threadIdx.x / kWave) > U / kWave) return;
   const int64_t row0 = row_splits[b];
   if (TILED) {
     if (blockIdx.y == 0)
@@ -1083,40 +1094,48 @@ static int launch_alpha_beta(const float *lp, const int32_t *logit_lengths,
   if (max_u1 > OT_MAX_U1) return OT_E_TOO_LONG;
   if (utt_begin == utt_end) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // more columns than a workgroup has threads: column tiles, one after the other
+  // One workgroup per (utterance, direction) with a thread per column, up to
+  // OT_LATTICE_TILE columns.  A batch with longer utterances gets two launches over the same
+  // grid: this one for the utterances that fit (each workgroup looks at its own U), and a
+  // second in which a workgroup of OT_LATTICE_TILE threads sweeps its utterance's columns
+  // tile by tile, so that one long utterance does not move the whole batch to that kernel.
   const bool tiled = max_u1 > OT_LATTICE_TILE;
   const int threads = tiled ? OT_LATTICE_TILE : ((max_u1 + kWave - 1) / kWave) * kWave;
   const dim3 grid((unsigned)(utt_end - utt_begin), 2), block((unsigned)threads);
   const bool multi = threads > kWave;
   const int nwaves = threads / kWave;
-  if (!one_sym_per_frame && nwaves >= 3 && !tiled) {
+  if (!one_sym_per_frame && nwaves >= 3) {
     // staging rings: (8 + 4) bytes per lane and group row
     const int G = nwaves <= 4 ? 16 : nwaves <= 9 ? 8 : 4;
     const size_t lds = (size_t)nwaves * G * kWave * 12;
 #define OT_LAUNCH_DPS(G_, THREADS_)                                                             \
   hipLaunchKernelGGL((alpha_beta_staged_kernel<G_, THREADS_>), grid, block, lds, s, lp,         \
                      logit_lengths, target_lengths, row_splits, utt_begin, alpha, beta,         \
-                     scores_alpha, scores_beta, guard_n, guard_rows)
+                     scores_alpha, scores_beta, max_u1, guard_n, guard_rows)
     if (G == 16) OT_LAUNCH_DPS(16, 256);
     else if (G == 8) OT_LAUNCH_DPS(8, 576);
     else OT_LAUNCH_DPS(4, 1024);
 #undef OT_LAUNCH_DPS
-    return launch_status();
-  }
-#define OT_LAUNCH_DP(OSF_, MULTI_, TILED_)                                                      \
-  hipLaunchKernelGGL((alpha_beta_kernel<OSF_, MULTI_, TILED_>), grid, block, 0, s, lp,          \
-                     logit_lengths, target_lengths, row_splits, utt_begin, alpha, beta,         \
-                     scores_alpha, scores_beta, tiled ? max_u1 : threads, guard_n, guard_rows)
-  if (one_sym_per_frame) {
-    if (tiled) OT_LAUNCH_DP(true, true, true);
-    else if (multi) OT_LAUNCH_DP(true, true, false);
-    else OT_LAUNCH_DP(true, false, false);
   } else {
-    if (tiled) OT_LAUNCH_DP(false, true, true);
-    else if (multi) OT_LAUNCH_DP(false, true, false);
-    else OT_LAUNCH_DP(false, false, false);
-  }
+#define OT_LAUNCH_DP(OSF_, MULTI_)                                                              \
+  hipLaunchKernelGGL((alpha_beta_kernel<OSF_, MULTI_, false>), grid, block, 0, s, lp,           \
+                     logit_lengths, target_lengths, row_splits, utt_begin, alpha, beta,         \
+                     scores_alpha, scores_beta, max_u1, guard_n, guard_rows)
+    if (one_sym_per_frame) {
+      if (multi) OT_LAUNCH_DP(true, true); else OT_LAUNCH_DP(true, false);
+    } else {
+      if (multi) OT_LAUNCH_DP(false, true); else OT_LAUNCH_DP(false, false);
+    }
 #undef OT_LAUNCH_DP
+  }
+  int rc = launch_status();
+  if (rc || !tiled) return rc;
+#define OT_LAUNCH_TILED(OSF_)                                                                   \
+  hipLaunchKernelGGL((alpha_beta_kernel<OSF_, true, true>), grid, dim3(OT_LATTICE_TILE), 0, s,  \
+                     lp, logit_lengths, target_lengths, row_splits, utt_begin, alpha, beta,     \
+                     scores_alpha, scores_beta, max_u1, guard_n, guard_rows)
+  if (one_sym_per_frame) OT_LAUNCH_TILED(true); else OT_LAUNCH_TILED(false);
+#undef OT_LAUNCH_TILED
   return launch_status();
 }
 

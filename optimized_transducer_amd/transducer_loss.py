@@ -12,7 +12,12 @@ Differences from the reference that do not change results:
   makes a full pass);
 * ``backward`` returns a fresh alias of the gradient buffer, so that autograd
   can adopt it as ``logits.grad`` without the (rows, V) copy the reference's
-  shared tensor object forces when ``logits`` is a leaf;
+  shared tensor object forces when ``logits`` is a leaf; a further backward
+  through the same graph (``retain_graph=True``), which the reference answers
+  with ``ctx.grad.mul_(loss_grad)`` once more (transducer_loss.py:160-162), gets
+  a copy of the buffer times ``loss_grad``, the copy being made then and not
+  before (it raises if the buffer was changed in place in between, e.g. by
+  ``logits.grad.zero_()``, which the reference's private copy would survive);
 * ``TransducerLoss.__init__`` calls ``super().__init__()`` so the module can
   actually be called (the reference's class omits it, transducer_loss.py:173-188).
 
@@ -118,19 +123,25 @@ class TransducerLossFunction(torch.autograd.Function):
                 loss_grad=factor,
             )
             return (grad,) + no_grads
-        # Hand autograd a fresh alias of the gradient buffer and drop ours: when
-        # `logits` is a leaf, autograd then adopts the buffer as logits.grad
-        # instead of cloning (rows, V) floats because others still hold it.
-        # The buffer is then autograd's (it may accumulate into it), so a second
-        # backward through the same graph (retain_graph=True), which the reference
-        # answers with the same tensor again (transducer_loss.py:160-162), is refused.
+        # Hand autograd a fresh alias of the gradient buffer: when `logits` is a leaf,
+        # autograd then adopts the buffer as logits.grad instead of cloning (rows, V)
+        # floats because this object still holds the tensor.  From then on the buffer is
+        # shared with autograd, which may accumulate into it.  A further backward through
+        # the same graph (retain_graph=True), which the reference answers with
+        # ctx.grad.mul_(loss_grad) once more (transducer_loss.py:160-162), therefore works
+        # on a copy, made only then; the version counter, which every alias shares, tells
+        # whether the buffer still holds what the previous backward returned.
         if ctx.grad is None:
-            raise RuntimeError(
-                "backward through transducer_loss runs once: the gradient buffer was handed "
-                "to autograd by the first backward (call transducer_loss again instead of "
-                "retain_graph=True)")
-        grad = ctx.grad.detach()
-        ctx.grad = None
+            return (None,) + no_grads
+        if getattr(ctx, "handed_version", None) is not None:
+            if ctx.grad._version != ctx.handed_version:
+                raise RuntimeError(
+                    "transducer_loss: the gradient buffer that an earlier backward handed to "
+                    "autograd has been modified in place since (for example by "
+                    "logits.grad.zero_()); call transducer_loss again instead of a second "
+                    "backward through the same graph")
+            ctx.grad = ctx.grad.clone()
+        grad = ctx.grad
         if (
             loss_grad.is_cuda
             and loss_grad.device == grad.device
@@ -140,7 +151,10 @@ class TransducerLossFunction(torch.autograd.Function):
         ):
             _optimized_transducer.scale_by_device_scalar_(grad, loss_grad.detach().contiguous())
         else:
-            grad.mul_(loss_grad)
+            with torch.no_grad():
+                grad.mul_(loss_grad)
+        ctx.handed_version = grad._version
+        grad = grad.detach()
         return (grad,) + no_grads
 
 

@@ -57,6 +57,16 @@ def lattice_noise_tolerance(ref_grad, loss_per_row, mag, k=NOISE_K, scale=1.0):
     return min(scale, 1.0) * ATOL + scale * (RTOL * np.abs(ref_grad) + noise)
 
 
+def oracle_noise_unit(x, targets, T, U, blank, fls, osf):
+    """(scores, fp32 gradient, per-entry noise unit) from one run of the fp32 oracle: the
+    unit is one float32 rounding of an entry's exponent, eps * |log-likelihood of the
+    utterance| * (sum of the entry's exponentials); lattice_noise_tolerance allows
+    NOISE_K of them on top of the north-star tolerance."""
+    s, g, mag = oracle.compute_transducer_loss(np.ascontiguousarray(x).copy(), targets, T, U, blank,
+                                               fls, osf, return_magnitude=True)
+    return s, g, EPS32 * np.abs(per_row(s, T, U))[:, None] * mag
+
+
 def oracle_tolerance(x, targets, T, U, blank, fls, osf, scale=1.0, k=NOISE_K):
     """(scores, unscaled fp32 gradient, elementwise bound for `scale` x that gradient)
     from one run of the fp32 oracle."""

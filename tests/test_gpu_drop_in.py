@@ -123,15 +123,35 @@ def test_padding_of_minus_one_is_accepted_and_negative_ids_that_are_read_are_not
                            torch.from_numpy(U), 0, False)
 
 
-def test_second_backward_is_refused_with_a_message(device):
+@pytest.mark.parametrize("fls", [False, True])
+def test_second_backward_through_the_same_graph(fls, device):
+    # the reference's backward returns ctx.grad.mul_(loss_grad) every time it is called
+    # (transducer_loss.py:158-170), so with retain_graph=True a leaf accumulates
+    # g * w1 + g * w1 * w2.  Here the first backward hands the buffer itself to autograd
+    # (no (rows, V) copy) and only a further backward copies.
     import optimized_transducer_amd as ot
     rng = np.random.default_rng(6)
     T, U, tg, x = helpers.random_batch(rng, 3, 10, 4, 9)
+    if fls:
+        x = helpers.log_softmax32(x)
+    _, g = oracle.compute_transducer_loss(x.copy(), tg, T, U, 0, fls, False)
+    g = g / len(T)
     logits = torch.from_numpy(x).to(device).requires_grad_(True)
     loss = ot.transducer_loss(logits, torch.from_numpy(tg).to(device), torch.from_numpy(T).to(device),
-                              torch.from_numpy(U).to(device), 0, False)
+                              torch.from_numpy(U).to(device), 0, fls)
+    (loss * 0.5).backward(retain_graph=True)
+    first = logits.grad
+    if not fls:
+        assert first.data_ptr() == logits.data_ptr()   # adopted, not cloned
+    assert np.allclose(first.cpu().numpy(), 0.5 * g, rtol=RTOL, atol=ATOL)
+    (loss * 3.0).backward(retain_graph=True)
+    assert logits.grad.data_ptr() == first.data_ptr()   # accumulated in place
+    assert np.allclose(logits.grad.cpu().numpy(), (0.5 + 0.5 * 3.0) * g, rtol=RTOL, atol=2e-5)
+    # a buffer that was changed in place since it was handed over cannot be returned again
+    logits.grad = None
     loss.backward(retain_graph=True)
-    with pytest.raises(RuntimeError, match="runs once"):
+    logits.grad.zero_()
+    with pytest.raises(RuntimeError, match="modified in place"):
         loss.backward()
 
 

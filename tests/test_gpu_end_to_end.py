@@ -498,6 +498,14 @@ FULL = [
 ]
 
 
+# gradient against the fp32 oracle: every entry within rel 1e-5 / abs 1e-5 ...
+PLAIN_TOLERANCE = ("asr_logsoftmax_modified", "ragged", "ragged_modified")
+# ... or at least this share of the entries, none further than NOISE_UNITS_MAX roundings of
+# its exponent
+NOISE_LIMITED = {"asr": 0.9999, "largevocab": 0.999999}
+NOISE_UNITS_MAX = helpers.NOISE_K  # measured: 1.0 to 2.4 over the six workloads
+
+
 @pytest.mark.parametrize("api", ["cabi", "python"])
 @pytest.mark.parametrize("name,make", FULL, ids=[f[0] for f in FULL])
 def test_full_size_workloads(name, make, api, device):
@@ -526,29 +534,37 @@ def test_full_size_workloads(name, make, api, device):
         assert int(splits[-2]) * w.V < 2 ** 31 < int(splits[-1]) * w.V
     xs = torch.cat([x[splits[b]:splits[b + 1]] for b in pick]).cpu().numpy()
     tgs = np.ascontiguousarray(tg[pick][:, :max(int(U[pick].max()), 0)])
-    s32, g32, tol = helpers.oracle_tolerance(xs, tgs, T[pick], U[pick], w.blank, fls, osf)
+    # the workload's own reduction: "mean" multiplies the gradient by 1/N (transducer_loss.py:150)
+    scale = 1.0 / len(T) if w.reduction == "mean" else 1.0
+    s32, g32, unit = helpers.oracle_noise_unit(xs, tgs, T[pick], U[pick], w.blank, fls, osf)
+    g32 *= np.float32(scale)
+    unit *= np.float32(scale)
+    plain = ATOL + RTOL * np.abs(g32)
+    # the absolute part shrinks with the scale, so that the bound keeps its power for "mean"
+    tol = min(scale, 1.0) * ATOL + RTOL * np.abs(g32) + helpers.NOISE_K * unit
     if huge:  # no float64 run at this size (memory, time)
         s64, g64 = s32, None
     else:
         s64, g64 = oracle.compute_transducer_loss(xs.copy(), tgs, T[pick], U[pick], w.blank, fls,
                                                   osf, dtype=np.float64)
+        g64 *= scale
 
     work = x.clone()
     if api == "cabi":
         scores, grad, st = cabi.transducer_loss(work, dtg, dT, dU, w.blank, fls, osf, max_u1,
-                                                grad=("new" if fls else "inplace"))
+                                                grad_scale=scale, grad=("new" if fls else "inplace"))
         assert st.sum_tu == total and st.targets_max == tg.max() and st.target_len_max == U.max()
     else:
         scores, _ = ext.compute_transducer_loss(
             logits=x.clone(), targets=dtg, logit_lengths=dT, target_lengths=dU, blank=w.blank,
             from_log_softmax=fls, one_sym_per_frame=osf)
         work.requires_grad_(True)
-        loss = ot.transducer_loss(work, dtg, dT, dU, w.blank, fls, osf, "sum")
+        loss = ot.transducer_loss(work, dtg, dT, dU, w.blank, fls, osf, w.reduction)
         loss.backward()
         grad = work.grad
         work = work.detach()
-        # loss = -sum of the per-utterance log-likelihoods (transducer_loss.py:145-147)
-        want_loss = -float(scores.double().sum())
+        # loss = -sum or -mean of the per-utterance log-likelihoods (transducer_loss.py:145-147)
+        want_loss = -scale * float(scores.double().sum())
         assert abs(loss.item() - want_loss) <= 1e-6 * abs(want_loss), (loss.item(), want_loss)
     scores_np = scores.cpu().numpy()
     assert np.isfinite(scores_np).all()
@@ -558,14 +574,31 @@ def test_full_size_workloads(name, make, api, device):
     assert np.allclose(got_s, s32, rtol=RTOL, atol=ATOL), np.abs(got_s - s32).max()
     err = np.abs(got_g - g32)
     assert (err <= tol).all(), (err.max(), (err / tol).max())
+    # The measured record per workload, pinned.  With the 1/N of their "mean" reduction the
+    # log-softmax workload, the large vocabulary and the ragged batches meet the plain
+    # rel 1e-5 / abs 1e-5 on every entry or all but a few in 10^7; on the long lattices of the
+    # "sum" workload, with |log-likelihood| of 2-3 thousand and no 1/N, a few entries in 10^5
+    # differ by some roundings of their exponent (eps * |log-likelihood| * the entry's
+    # exponentials; entries with a unit below 1e-30 are denormal results, which the GPU
+    # flushes to zero).
+    within = err <= plain
+    ok = unit > 1e-30
+    units = (err[ok] / unit[ok]).max() if ok.any() else 0.0
+    print("parity %s/%s (%s): max |err| = %.3g, share within rel/abs 1e-5 = %.8f, largest error = %.2f "
+          "noise units" % (name, api, w.reduction, err.max(), within.mean(), units))
+    if name in PLAIN_TOLERANCE:
+        assert within.all(), (name, err.max(), 1.0 - within.mean())
+    elif name in NOISE_LIMITED:
+        assert within.mean() >= NOISE_LIMITED[name] and units <= NOISE_UNITS_MAX, (name, within.mean(), units)
+    del within, ok
     # float64 arbiter: no further from the exact gradient than the fp32 reference arithmetic
     if g64 is not None:
-        assert np.abs(got_g - g64).max() <= 2 * np.abs(g32 - g64).max() + 1e-6
+        assert np.abs(got_g - g64).max() <= 2 * np.abs(g32 - g64).max() + 1e-6 * scale
     del xs, g32, g64, got_g
 
     # size-independent properties over the whole batch
     if fls:
-        occ = -grad.sum(1)  # node occupancies
+        occ = -grad.sum(1) / scale  # node occupancies
         assert (occ >= -1e-6).all()
         assert (occ <= 1 + 64 * helpers.EPS32 * np.abs(scores_np).max()).all()
         # occupancies of one frame (modified) / all frames (standard) add up per utterance
@@ -584,5 +617,5 @@ def test_full_size_workloads(name, make, api, device):
     # same bits on a second run (no atomics, no data races)
     work2 = x.clone()
     scores2, grad2, _ = cabi.transducer_loss(work2, dtg, dT, dU, w.blank, fls, osf, max_u1,
-                                             grad=("new" if fls else "inplace"))
+                                             grad_scale=scale, grad=("new" if fls else "inplace"))
     assert torch.equal(scores2, scores) and torch.equal(grad2, grad)

@@ -38,6 +38,10 @@ def _cases():
             ("two_waves_V64", 3, 90, 100, 64, 1, False), ("two_waves_V64_mod", 3, 120, 100, 64, 1, True),
             ("five_waves_V8", 2, 40, 300, 8, 0, False), ("five_waves_V8_mod", 2, 330, 300, 8, 0, True),
             ("many_utts_V16", 300, 6, 4, 16, 0, False),
+            # beyond the 1024 utterances up to which a workgroup finds its utterances by a
+            # wave-parallel count
+            ("thousands_of_utts_V16", 3000, 5, 3, 16, 2, False),
+            ("thousands_of_utts_V12_mod", 2500, 6, 3, 12, 0, True),
             ("V1000", 4, 12, 6, 1000, 999, False), ("V5000", 2, 7, 4, 5000, 0, False),
             ("V5004_mod", 2, 7, 4, 5004, 17, True), ("V2049", 2, 5, 3, 2049, 0, False)]:
         T, U, tg, x = helpers.random_batch(rng, N, tmax, umax, V, one_sym_per_frame=osf)
