@@ -40,7 +40,7 @@ extern "C" {
 #define OT_LATTICE_TILE 1024
 /* Largest max_u1 = max_b(U_b)+1 accepted.  What really bounds an utterance is
  * that its cells are addressed with 32-bit byte offsets:
- * (T_b + 1300) * (U_b + 1) < 2^29. */
+ * (T_b + 1300) * (U_b + 1) < 2^28. */
 #define OT_MAX_U1 (1 << 18)
 
 /* Batch facts gathered on the device by ot_row_splits; the host-side argument
@@ -109,7 +109,7 @@ int ot_log_probs_range(const float *logits, const int32_t *targets,
  * scores_beta[b] = beta(0,0); both are log-likelihoods.  Cells outside the
  * band of the one-symbol-per-frame lattice (uninitialised in the reference)
  * are -inf.  max_u1 = max_b(U_b)+1 sizes the workgroup; must be <= OT_MAX_U1,
- * and every utterance must satisfy (T_b + 1300) * (U_b + 1) < 2^29. */
+ * and every utterance must satisfy (T_b + 1300) * (U_b + 1) < 2^28. */
 int ot_alpha_beta(const float *lp, const int32_t *logit_lengths,
                   const int32_t *target_lengths, const int32_t *row_splits,
                   int32_t N, int32_t max_u1, int32_t one_sym_per_frame,

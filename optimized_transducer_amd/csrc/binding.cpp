@@ -395,7 +395,7 @@ std::pair<torch::Tensor, torch::optional<torch::Tensor>> compute_impl(
               st.logit_len_min, " and ", st.target_len_min);
   const int32_t max_u1 = st.target_len_max + 1;
   // the lattice kernel addresses one utterance's cells with 32-bit byte offsets
-  TORCH_CHECK(((int64_t)st.logit_len_max + 1300) * max_u1 < ((int64_t)1 << 29),
+  TORCH_CHECK(((int64_t)st.logit_len_max + 1300) * max_u1 < ((int64_t)1 << 28),
               "an utterance with T = ", st.logit_len_max, " and up to ", max_u1,
               " lattice columns is too large for the lattice kernel");
 

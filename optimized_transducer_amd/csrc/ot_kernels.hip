@@ -624,12 +624,13 @@ __device__ __forceinline__ void lattice_sweep_staged(const float *__restrict__ l
 // what its memory safety rests on itself and does nothing otherwise (guard_n = N, or 0
 // for a launch after validation): the rows of the batch add up to the size of the
 // arrays, every utterance has T >= 1 and 0 <= U < the columns the launch was sized for,
-// and its cells fit 32-bit byte offsets.
+// and the byte offsets of its cells (8 bytes each, rows up to 1300 beyond either end
+// included) stay below 2^31.
 __device__ __forceinline__ bool lattice_guard_ok(const int32_t *__restrict__ row_splits, int guard_n,
                                                  int64_t guard_rows, int T, int U, int max_u1) {
   if (guard_n <= 0) return true;
   return (int64_t)row_splits[guard_n] == guard_rows && T >= 1 && U >= 0 && U < max_u1 &&
-         ((int64_t)T + 1300) * ((int64_t)U + 1) < ((int64_t)1 << 29);
+         ((int64_t)T + 1300) * ((int64_t)U + 1) < ((int64_t)1 << 28);
 }
 
 template <int G, int THREADS>
@@ -654,6 +655,287 @@ __global__ __launch_bounds__(THREADS) void alpha_beta_staged_kernel(
     lattice_sweep_staged<false, G>(lp, T, U, row0, alpha, scores_alpha + b, s_ring, s_stage);
   else
     lattice_sweep_staged<true, G>(lp, T, U, row0, beta, scores_beta + b, s_ring, s_stage);
+}
+
+// ---------------------------------------------------------------------------
+// Lattices of up to kServedWaves * 64 columns: the recursion with memory waves beside it.
+//
+// The waves that walk the recursion ("compute waves", one lane per column as above)
+// execute no global memory instruction at all.  Every 64 columns have two more waves:
+//   - a loader, which fetches the lp cells of the steps ahead (kLoadAhead chunks of
+//     kChunk steps in flight, in registers) and puts each cell into an LDS ring at
+//     [step mod 2*kChunk][lane], i.e. where the compute lane that needs it at that step
+//     reads it with a compile-time offset;
+//   - a storer, which takes the results of the chunk before out of a second ring of the
+//     same shape and writes them to alpha/beta.
+// On the anti-diagonal wavefront the 64 cells of a step lie in 64 different rows of the
+// arrays, which is what the one-thread-per-column sweep pays for from two waves on (64
+// cache lines per load and per store instruction).  A chunk of 16 steps of a wave covers a
+// parallelogram of 79 rows with 16 consecutive columns each; loader and storer walk it
+// row-wise, four rows of 16 columns per instruction, and the LDS rings do the skewing.
+// Their latencies (and those of a busy memory system) stay out of the recursion as long
+// as the loader is kLoadAhead chunks ahead; when it is not, it arrives late at the chunk's
+// barrier and everyone waits for it.
+// One barrier per chunk orders everything: the loader writes chunk c+1's slots while the
+// compute wave reads chunk c's, the storer reads chunk c-1's results while chunk c's are
+// written to the other half of the ring.
+// On the one-symbol-per-frame lattice all lanes of a wave are in the same row in every
+// step; the band (cells outside it are -inf) is applied to the lp values by the loader:
+//   alpha: the blank arc out of a cell with t - u >= T-1-U leaves the band, so that
+//          cell's blank term becomes -inf (the final blank is read from memory, not here);
+//   beta : both terms of a cell outside the band become -inf.
+// The arithmetic of a step is that of lattice_sweep, bit for bit (natural logarithms,
+// log_add with the reference's threshold).  Keeping the values as base-2 logarithms would
+// take three instructions out of the step's dependent chain (measured: 57 instead of 64 ns
+// per step at two waves), but every rounding then falls differently from the reference's,
+// and the gradient of a long lattice ends up five times further from the reference's
+// (2.5e-3 instead of 4.9e-4 at 2 x 10^3 nats) although no further from the exact one.
+// ---------------------------------------------------------------------------
+constexpr int kServedWaves = 4;            // compute waves per workgroup, 3 waves per 64 columns
+// chunks of lp in flight per loader (20 loads each, at most 63 may be outstanding); two
+// where three waves share a SIMD's registers
+constexpr int load_ahead(int compute_waves) { return compute_waves <= 2 ? 3 : 2; }
+constexpr int kRingSlots = kChunk + 1;     // slots per half: one per step + a dummy for masked lanes
+
+template <int C>
+struct ServedLds {
+  float ring[C][kRing + kChunk];                  // values that cross a wave boundary
+  f32x2 lp[C][2][kRingSlots][kWave];              // lp cells by (step mod 32, lane)
+  float out[C][2][kRingSlots][kWave];             // results by (step mod 32, lane)
+};
+
+// Which cell instruction k of a loader / storer lane handles in a chunk: step dn within
+// the chunk and compute lane j it belongs to (j outside [0, 64) or a column beyond U: none),
+// and the lattice row at chunk 0; rows advance by kChunk per chunk (backwards for beta).
+template <bool BETA, bool OSF>
+struct ServedCells {
+  static constexpr int kInstr = OSF ? kChunk : 20;
+  int w, wlast, T, U, lane;
+  __device__ __forceinline__ void cell(int k, int &dn, int &j, int &t0) const {
+    const int r = lane >> 4, c = lane & 15;
+    if (OSF) {
+      dn = k;
+      j = lane;
+      const int tt = k - (BETA ? (wlast - w) : w) * kLag;  // steps since the wave's start
+      t0 = BETA ? T - 1 - tt : tt;
+    } else if (!BETA) {
+      // delay = 64w + j + 16w, t + j = n - 80w
+      dn = c;
+      j = 64 - 4 * k - r + c;
+      t0 = -80 * w - 64 + 4 * k + r;
+    } else {
+      // mirrored: delay = (U - 64w - j) + 16(wlast - w)
+      dn = 15 - c;
+      j = 4 * k + r - 15 + c;
+      const int tt = -(U - 64 * w) - (wlast - w) * kLag + 4 * k + r;
+      t0 = T - 1 - tt;
+    }
+  }
+};
+
+template <bool BETA, bool OSF, int C>
+__device__ __forceinline__ void served_sweep(const float *__restrict__ lp, int T, int U,
+                                             int64_t row0, float *__restrict__ out,
+                                             float *__restrict__ score, ServedLds<C> &lds) {
+  const int wid = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int role = wid / C, w = wid - role * C;  // 0 compute, 1 loader, 2 storer
+  const int U1 = U + 1;
+  const int wlast = U / kWave;
+  if (w > wlast) return;  // no columns: a barrier only waits for the waves that have not ended
+  const int nsteps = (OSF ? T : T + U) + wlast * kLag;
+  const int nchunks = (nsteps + kChunk - 1) / kChunk;
+  const int diff = T - 1 - U;  // width of the one-symbol-per-frame band; negative: infeasible
+  const unsigned cells = (unsigned)T * (unsigned)U1;
+  // Offset of a lane that has no cell.  Offsets move by one chunk of rows per chunk, all
+  // strides of an utterance add up to less than 2^31 bytes (lattice_guard_ok), and the
+  // arrays are shorter than that: counting up from 2^31 (alpha) or down from 2^32 - 1
+  // (beta) never reaches them.  Rows before the first or behind the last wrap around to
+  // offsets beyond the arrays in the same way.
+  constexpr unsigned kOob = BETA ? 0xFFFFFFFFu : 0x80000000u;
+  constexpr int kLoadAhead = load_ahead(C);
+
+  if (role == 0) {
+    // ---- the recursion: LDS in, LDS out ----
+    const int u = w * kWave + lane;
+    const bool column = u <= U;
+    const int src_wave = BETA ? w + 1 : w - 1;
+    const bool has_src = C > 1 && src_wave >= 0 && src_wave <= wlast;
+    const int src_ok = has_src ? src_wave : w;
+    const int edge_lane = BETA ? 0 : kWave - 1;
+    float *const ring_dst = &lds.ring[w][(lane == edge_lane) ? 0 : kRing];
+    const int ring_mask = (lane == edge_lane) ? (kRing - 1) : 0;
+    const int ering_step = BETA ? (kWave - 1 - lane) : lane;
+    float own = (column && u == (BETA ? U : 0) && !(OSF && diff < 0)) ? 0.f : OT_NEG_INF;
+    float nb = OT_NEG_INF;
+    lds_barrier();  // chunk 0 of lp is in the ring
+    for (int c = 0; c < nchunks; ++c) {
+      const int n = c * kChunk, half = c & 1;
+      const f32x2 *const lp_rd = &lds.lp[w][half][0][lane];
+      float *const out_wr = &lds.out[w][half][0][lane];
+      float ering = OT_NEG_INF;
+      float *ring_wr = nullptr;
+      if (C > 1) {
+        const int s = n - 1 - kLag + ering_step;
+        const float v = lds.ring[src_ok][s & (kRing - 1)];
+        ering = (has_src && ering_step < kChunk && s >= 0) ? v : OT_NEG_INF;
+        ring_wr = ring_dst + (n & ring_mask);
+      }
+      f32x2 q[kChunk];
+#pragma unroll
+      for (int i = 0; i < kChunk; ++i) q[i] = lp_rd[i * kWave];
+#pragma unroll
+      for (int i = 0; i < kChunk; ++i) {
+        const f32x2 l = q[i];
+        const float in = BETA ? wave_shift_down(nb, ering) : wave_shift_up(nb, ering);
+        if (C > 1) ering = BETA ? dpp_mov<kDppWaveShr1>(ering) : dpp_mov<kDppWaveShl1>(ering);
+        const float a = BETA ? log_add(own + l.x, in + l.y) : log_add(own, in);
+        out_wr[i * kWave] = a;
+        if (BETA) {
+          own = nb = a;
+        } else {
+          own = a + l.x;
+          nb = a + l.y;
+        }
+        if (C > 1) ring_wr[i] = nb;
+      }
+      lds_barrier();
+    }
+    // the utterance's score from the last cell of the recursion, which this lane computed
+    // in the last step (alpha: alpha(T-1,U) plus blank(T-1,U); beta: beta(0,0))
+    if (column && u == (BETA ? 0 : U)) {
+      const int nf = nsteps - 1;
+      const float af = lds.out[w][(nf / kChunk) & 1][nf & (kChunk - 1)][lane];
+      if (BETA) {
+        *score = af;
+      } else {
+        const int64_t last = row0 + (int64_t)cells - 1;
+        *score = af + lp[2 * last];
+      }
+    }
+    return;
+  }
+
+  // ---- memory waves: per-lane cell map, fixed over the chunks ----
+  using Cells = ServedCells<BETA, OSF>;
+  constexpr int KI = Cells::kInstr;
+  const Cells map{w, wlast, T, U, lane};
+  const int drow = BETA ? -kChunk : kChunk;  // rows per chunk
+  if (role == 1) {
+    const __amdgpu_buffer_rsrc_t lp_buf = make_buffer(lp + 2 * row0, cells * 8u);
+    unsigned off[KI];       // byte offset of the cell in chunk 0 (top bit set: no cell)
+    int slot[KI];           // element index in lds.lp[w][0], the dummy slot for no cell
+    int tu[KI];             // t - u at chunk 0 (one-symbol-per-frame band)
+#pragma unroll
+    for (int k = 0; k < KI; ++k) {
+      int dn, j, t0;
+      map.cell(k, dn, j, t0);
+      const int u = w * kWave + j;
+      const bool lane_ok = j >= 0 && j < kWave;
+      // a compute lane without a column (u > U) still reads its slots: it gets zeros, as
+      // the out-of-range loads of rows outside the lattice give them, never stale LDS
+      off[k] = (lane_ok && u <= U) ? (unsigned)(t0 * U1 + u) * 8u : kOob;
+      slot[k] = lane_ok ? dn * kWave + j : kChunk * kWave + lane;
+      tu[k] = t0 - u;
+    }
+    const unsigned dchunk = (unsigned)(drow * U1) * 8u;
+    f32x2 reg[kLoadAhead][KI];
+    auto issue = [&](f32x2(&r)[KI]) {
+#pragma unroll
+      for (int k = 0; k < KI; ++k) {
+        r[k] = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(lp_buf, off[k], 0, 0));
+        off[k] += dchunk;
+      }
+    };
+    // c: the chunk these cells belong to
+    auto deposit = [&](const f32x2(&r)[KI], int c) {
+      f32x2 *const base = &lds.lp[w][c & 1][0][0];
+#pragma unroll
+      for (int k = 0; k < KI; ++k) {
+        f32x2 v = r[k];
+        if (OSF) {
+          const int d = tu[k] + c * drow;  // t - u of this cell
+          if (BETA) {
+            const bool inband = (unsigned)d <= (unsigned)diff && diff >= 0;
+            v.x = inband ? v.x : OT_NEG_INF;
+            v.y = inband ? v.y : OT_NEG_INF;
+          } else {
+            v.x = (d >= diff) ? OT_NEG_INF : v.x;
+          }
+        }
+        base[slot[k]] = v;
+      }
+    };
+#pragma unroll
+    for (int a = 0; a < kLoadAhead; ++a) issue(reg[a]);
+    deposit(reg[0], 0);
+    lds_barrier();
+    // chunk c: fetch chunk c + kLoadAhead into the registers chunk c has left, hand chunk
+    // c + 1 to the ring (its half was read for the last time before the barrier above)
+    for (int c = 0; c < nchunks; c += kLoadAhead) {
+#pragma unroll
+      for (int a = 0; a < kLoadAhead; ++a) {
+        if (c + a < nchunks) {
+          issue(reg[a]);
+          deposit(reg[(a + 1) % kLoadAhead], c + a + 1);
+          lds_barrier();
+        }
+      }
+    }
+    return;
+  }
+
+  {
+    const __amdgpu_buffer_rsrc_t out_buf = make_buffer(out + row0, cells * 4u);
+    unsigned off[KI];
+    int slot[KI];
+#pragma unroll
+    for (int k = 0; k < KI; ++k) {
+      int dn, j, t0;
+      map.cell(k, dn, j, t0);
+      const int u = w * kWave + j;
+      const bool ok = j >= 0 && j < kWave && u <= U;
+      off[k] = ok ? (unsigned)(t0 * U1 + u) * 4u : kOob;
+      slot[k] = ok ? dn * kWave + j : kChunk * kWave + lane;
+    }
+    const unsigned dchunk = (unsigned)(drow * U1) * 4u;
+    // results of chunk c, once the barrier behind it has been passed
+    auto drain = [&](int c) {
+      const float *const base = &lds.out[w][c & 1][0][0];
+      float v[KI];
+#pragma unroll
+      for (int k = 0; k < KI; ++k) v[k] = base[slot[k]];
+#pragma unroll
+      for (int k = 0; k < KI; ++k) {
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v[k]), out_buf, off[k], 0, 0);
+        off[k] += dchunk;
+      }
+    };
+    lds_barrier();
+    for (int c = 0; c < nchunks; ++c) {
+      if (c) drain(c - 1);
+      lds_barrier();
+    }
+    drain(nchunks - 1);
+  }
+}
+
+template <bool OSF, int C>
+__global__ __launch_bounds__(3 * C * kWave) void alpha_beta_served_kernel(
+    const float *__restrict__ lp, const int32_t *__restrict__ logit_lengths,
+    const int32_t *__restrict__ target_lengths, const int32_t *__restrict__ row_splits,
+    int utt_begin, float *__restrict__ alpha, float *__restrict__ beta,
+    float *__restrict__ scores_alpha, float *__restrict__ scores_beta, int max_u1, int guard_n,
+    int64_t guard_rows) {
+  __shared__ ServedLds<C> lds;
+  const int b = utt_begin + blockIdx.x;
+  const int T = logit_lengths[b], U = target_lengths[b];
+  if (!lattice_guard_ok(row_splits, guard_n, guard_rows, T, U, max_u1)) return;
+  if (T < 1 || U < 0 || U >= C * kWave) return;  // not an utterance of this launch
+  const int64_t row0 = row_splits[b];
+  if (blockIdx.y == 0)
+    served_sweep<false, OSF, C>(lp, T, U, row0, alpha, scores_alpha + b, lds);
+  else
+    served_sweep<true, OSF, C>(lp, T, U, row0, beta, scores_beta + b, lds);
 }
 
 // One sweep per tile of OT_LATTICE_TILE columns, in the order of the recursion (alpha:
@@ -1104,6 +1386,24 @@ static int launch_alpha_beta(const float *lp, const int32_t *logit_lengths,
   const dim3 grid((unsigned)(utt_end - utt_begin), 2), block((unsigned)threads);
   const bool multi = threads > kWave;
   const int nwaves = threads / kWave;
+  if (nwaves <= kServedWaves) {
+    // up to 256 columns: compute waves beside loader and storer waves
+#define OT_LAUNCH_SERVED(OSF_, C_)                                                              \
+  hipLaunchKernelGGL((alpha_beta_served_kernel<OSF_, C_>), grid, dim3(3 * C_ * kWave), 0, s,    \
+                     lp, logit_lengths, target_lengths, row_splits, utt_begin, alpha, beta,     \
+                     scores_alpha, scores_beta, max_u1, guard_n, guard_rows)
+#define OT_LAUNCH_SERVED_C(OSF_)                                                                \
+  switch (nwaves) {                                                                             \
+    case 1: OT_LAUNCH_SERVED(OSF_, 1); break;                                                   \
+    case 2: OT_LAUNCH_SERVED(OSF_, 2); break;                                                   \
+    case 3: OT_LAUNCH_SERVED(OSF_, 3); break;                                                   \
+    default: OT_LAUNCH_SERVED(OSF_, 4); break;                                                  \
+  }
+    if (one_sym_per_frame) { OT_LAUNCH_SERVED_C(true) } else { OT_LAUNCH_SERVED_C(false) }
+#undef OT_LAUNCH_SERVED_C
+#undef OT_LAUNCH_SERVED
+    return launch_status();
+  }
   if (!one_sym_per_frame && nwaves >= 3) {
     // staging rings: (8 + 4) bytes per lane and group row
     const int G = nwaves <= 4 ? 16 : nwaves <= 9 ? 8 : 4;
