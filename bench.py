@@ -448,6 +448,31 @@ def bench_project(args):
 
     elapsed, spread = timed_steps(torch, fused, K, W)
     elapsed_unfused, spread_unfused = timed_steps(torch, unfused, K, W)
+
+    # The whole training step of the joiner's tail: projection + loss forward and backward
+    # down to the gradients of x, weight and bias (the backward products are torch's own
+    # in both arrangements).
+    xg = x.clone().requires_grad_(True)
+    wg = wt.clone().requires_grad_(True)
+    bg = bias.clone().requires_grad_(True)
+
+    def whole_fused():
+        xg.grad = wg.grad = bg.grad = None
+        loss = ot.joiner_transducer_loss(xg, wg, bg, targets, T, U, w.blank, w.one_sym_per_frame,
+                                         "sum", float32_logits=f32_logits)
+        loss.backward()
+
+    def whole_unfused():
+        xg.grad = wg.grad = bg.grad = None
+        if f32_logits:
+            logits = torch.nn.functional.linear(xg.float(), wg.float(), bg)
+        else:
+            logits = torch.nn.functional.linear(xg, wg, bg.to(act))
+        loss = ot.transducer_loss(logits, targets, T, U, w.blank, False, w.one_sym_per_frame, "sum")
+        loss.backward()
+
+    elapsed_whole, spread_whole = timed_steps(torch, whole_fused, K, W)
+    elapsed_whole_unfused, spread_whole_unfused = timed_steps(torch, whole_unfused, K, W)
     flops = 2.0 * R * D * V  # of the real columns, padded or not
     out = {
         "metric": "utterances/sec joiner output projection (fused denominators) + transducer loss "
@@ -464,6 +489,13 @@ def bench_project(args):
         "unfused": {"ms_per_step": 1e3 * elapsed_unfused / K, "step_ms": spread_unfused,
                     "what": "torch (hipBLASLt) projection of the same operands, then the loss with "
                             "its own denominator pass"},
+        "whole_step": {
+            "what": "projection + loss forward and backward down to the gradients of x, weight and "
+                    "bias: joiner_transducer_loss(...).backward() against torch's linear (in float32 "
+                    "for float32 logits) followed by transducer_loss",
+            "fused_ms_per_step": 1e3 * elapsed_whole / K, "fused_step_ms": spread_whole,
+            "unfused_ms_per_step": 1e3 * elapsed_whole_unfused / K,
+            "unfused_step_ms": spread_whole_unfused},
     }
     ext.set_profiling(True)
     for _ in range(K):

@@ -413,6 +413,27 @@ int ot_joiner_project(const void *x, const void *weight, const float *bias,
                       void *logits, int32_t logits_dtype, float *den,
                       void *stream);
 
+/* Backward of that projection with respect to its parameters (no counterpart
+ * in the reference either: there autograd's Linear does it, README.md:176-177
+ * with the loss's gradient of cuda.cu:471-489 as input):
+ *     grad_weight[v, k] = sum_r grad_logits[r, v] * x[r, k]
+ *     grad_bias[v]      = sum_r grad_logits[r, v]
+ * on the matrix cores with float32 accumulation, the rows split into slices
+ * whose partial sums are added in a fixed order (same bits on every run);
+ * grad_weight is rounded once to `dtype`, grad_bias (may be NULL) is float32.
+ *
+ * grad_logits (rows, V) and x (rows, D) row-major of `dtype` (OT_DTYPE_F16 or
+ * OT_DTYPE_BF16), 16-byte aligned, V and D multiples of 8; rows up to 2^31-1;
+ * workspace: ot_joiner_weight_grad_workspace_bytes(rows, V, D) bytes, 16-byte
+ * aligned, contents irrelevant before and after.  OT_E_TOO_LONG when a slice of
+ * the rows is longer than 32-bit byte offsets address (rows * max(V, D) beyond
+ * about 2^35). */
+size_t ot_joiner_weight_grad_workspace_bytes(int64_t rows, int32_t V, int32_t D);
+int ot_joiner_weight_grad(const void *grad_logits, const void *x, int32_t dtype,
+                          int64_t rows, int32_t V, int32_t D, void *workspace,
+                          size_t workspace_bytes, void *grad_weight,
+                          float *grad_bias, void *stream);
+
 /* The gather step of ot_log_probs for denominators that are already known
  * (ComputeLogProbs, cpu.cc:52-100, without the log-sum-exp in front of it):
  * lp[row] = (logits[row, blank], logits[row, target(row)]) - den[row];

@@ -26,7 +26,8 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-ffp-contract=off", "-fno-fast-math", "-Wall",
 ]
-KERNEL_SOURCES = ("ot_kernels.hip", "ot_joiner.hip", "ot_half.hip", "ot_project.hip")
+KERNEL_SOURCES = ("ot_kernels.hip", "ot_joiner.hip", "ot_half.hip", "ot_project.hip",
+                  "ot_project_grad.hip")
 OBJ_DIR = os.path.join(HERE, "build")  # objects only; ignored by git
 
 

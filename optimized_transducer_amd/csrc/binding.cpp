@@ -801,6 +801,36 @@ std::pair<torch::Tensor, torch::Tensor> joiner_project(const torch::Tensor &x,
   return {logits, den};
 }
 
+// Gradient of that projection with respect to weight and bias (ot_joiner_weight_grad):
+// (grad_weight (V, D) of x's dtype, grad_bias (V) float32) from the gradient of the logits.
+std::pair<torch::Tensor, torch::Tensor> joiner_weight_grad(const torch::Tensor &grad_logits,
+                                                           const torch::Tensor &x) {
+  const int dtype = half_dtype(x);
+  TORCH_CHECK(dtype != OT_DTYPE_F32, "joiner_weight_grad takes float16 or bfloat16 x, got ", x.scalar_type());
+  TORCH_CHECK(x.is_cuda() && grad_logits.device() == x.device(), "grad_logits and x must be on one HIP device");
+  TORCH_CHECK(x.dim() == 2 && grad_logits.dim() == 2 && x.size(0) == grad_logits.size(0) &&
+                  grad_logits.scalar_type() == x.scalar_type() && x.is_contiguous() &&
+                  grad_logits.is_contiguous(),
+              "expect contiguous grad_logits (rows, V) and x (rows, D) of one dtype");
+  const int64_t rows = x.size(0), D = x.size(1), V = grad_logits.size(1);
+  TORCH_CHECK(rows > 0 && rows <= INT32_MAX && V > 0 && D > 0 && V % 8 == 0 && D % 8 == 0,
+              "joiner_weight_grad needs rows > 0 and V, D positive multiples of 8, got rows = ", rows,
+              ", V = ", V, ", D = ", D);
+  c10::hip::HIPGuardMasqueradingAsCUDA device_guard(x.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+  const size_t ws_bytes = ot_joiner_weight_grad_workspace_bytes(rows, (int32_t)V, (int32_t)D);
+  torch::Tensor workspace = torch::empty({(int64_t)ws_bytes}, x.options().dtype(torch::kUInt8));
+  torch::Tensor grad_w = torch::empty({V, D}, x.options());
+  torch::Tensor grad_b = torch::empty({V}, x.options().dtype(torch::kFloat));
+  {
+    ScopedTimer timer("joiner_weight_grad", stream);
+    OT_CHECK(ot_joiner_weight_grad(grad_logits.data_ptr(), x.data_ptr(), dtype, rows, (int32_t)V,
+                                   (int32_t)D, workspace.data_ptr(), ws_bytes, grad_w.data_ptr(),
+                                   grad_b.data_ptr<float>(), stream));
+  }
+  return {grad_w, grad_b};
+}
+
 PYBIND11_MODULE(_optimized_transducer, m) {
   m.doc() = "MI355X-native transducer loss (drop-in for optimized_transducer's extension module)";
 #ifdef OT_BUILT_WITH_TORCH
@@ -857,6 +887,9 @@ PYBIND11_MODULE(_optimized_transducer, m) {
         py::arg("float32_logits"),
         "logits = x @ weight.T + bias for float16 / bfloat16 x (rows, D) and weight (V, D) on the "
         "matrix cores, and their per-row log-sum-exp: returns (logits, denominators).");
+  m.def("joiner_weight_grad", &joiner_weight_grad, py::arg("grad_logits"), py::arg("x"),
+        "Backward of joiner_project in its parameters: (grad_logits.T @ x in x's dtype, "
+        "grad_logits.sum(0) in float32) for float16 / bfloat16 operands, float32 accumulation.");
   m.def("set_profiling", &set_profiling, py::arg("on"));
   m.def("set_overlap", &set_overlap, py::arg("on"),
         "Run the lattice kernel of one half of a large batch on a second stream while the "

@@ -118,16 +118,32 @@ class ProjectJoinerFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_logits, _grad_den):
-        # plain dense products: the library's kernels.  With a padded vocabulary the saved
-        # weight is the padded one and the incoming gradient is zero in the masked columns.
+        # With a padded vocabulary the saved weight is the padded one and the incoming
+        # gradient is zero in the masked columns.
         x, weight = ctx.saved_tensors
         V = ctx.V
         g = grad_logits if grad_logits.dtype == x.dtype else grad_logits.to(x.dtype)
+        # grad_x: a product with the contraction index running fastest in memory on one
+        # side, the kind the library's kernels are good at
         grad_x = g @ weight if ctx.needs_input_grad[0] else None
-        grad_w = (g.t() @ x)[:V] if ctx.needs_input_grad[1] else None
-        grad_b = None
-        if ctx.has_bias and ctx.needs_input_grad[2]:
-            grad_b = grad_logits.sum(0, dtype=torch.float32)[:V].to(ctx.bias_dtype)
+        want_w = ctx.needs_input_grad[1]
+        want_b = ctx.has_bias and ctx.needs_input_grad[2]
+        grad_w = grad_b = None
+        if (want_w or want_b) and g.shape[1] % 8 == 0 and x.shape[1] % 8 == 0:
+            # grad_W = g^T x and grad_b = sum of g's rows from one pass over g and x.  (The
+            # bias gradient is the sum of the 16-bit g here; with float32 logits that is g
+            # after its rounding to x's dtype, the same values grad_W is made of.)
+            g = g.contiguous()
+            gw, gb = _optimized_transducer.joiner_weight_grad(grad_logits=g, x=x)
+            if want_w:
+                grad_w = gw[:V]
+            if want_b:
+                grad_b = gb[:V].to(ctx.bias_dtype)
+        else:
+            if want_w:
+                grad_w = (g.t() @ x)[:V]
+            if want_b:
+                grad_b = grad_logits.sum(0, dtype=torch.float32)[:V].to(ctx.bias_dtype)
         return grad_x, grad_w, grad_b, None, None
 
 
@@ -159,8 +175,10 @@ def project_joiner(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
       ``logits.logsumexp(1)`` of exactly the stored values, taken from the
       accumulators.  Pass both to ``transducer_loss(logits, ..., from_log_softmax=False,
       denominators=denominators)``: the loss then reads the logits once, not twice.
-      Differentiable in ``x``, ``weight`` and ``bias`` (the backward products are
-      torch's own); ``denominators`` carries no gradient.
+      Differentiable in ``x``, ``weight`` and ``bias``: the gradients of ``weight`` and
+      ``bias`` come from this package's own kernel when V is a multiple of 8 (one pass over
+      the gradient of the logits and ``x``, float32 accumulation, the same bits on every
+      run), the gradient of ``x`` from torch's product; ``denominators`` carries no gradient.
     """
     if vocab_multiple is not None and (not isinstance(vocab_multiple, int) or vocab_multiple < 1):
         raise ValueError("project_joiner: vocab_multiple must be a positive integer or None, "

@@ -258,3 +258,16 @@ def project_joiner(x, weight, bias=None):
         out = out + b[None, :]
         mag = mag + np.abs(b)[None, :]
     return out, mag
+
+
+def project_joiner_weight_grad(grad_logits, x):
+    """Backward of that projection in its parameters, as autograd's Linear forms it
+    behind README.md:176-177: grad_weight = grad_logits^T x (V, D) and grad_bias = the
+    column sums of grad_logits (V), in float64, each with the sum of the absolute values
+    of its terms (the scale of the rounding error of a float32 accumulation in any
+    order)."""
+    g = np.asarray(grad_logits, dtype=np.float64)
+    x = np.asarray(x, dtype=np.float64)
+    gw = g.T @ x
+    gw_mag = np.abs(g).T @ np.abs(x)
+    return gw, gw_mag, g.sum(0), np.abs(g).sum(0)

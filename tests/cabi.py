@@ -285,6 +285,26 @@ def joiner_project(x, weight, bias, out_dtype, logits=None):
     return logits, den
 
 
+def joiner_weight_grad(grad_logits, x, want_bias=True, workspace_fill=None):
+    """(grad_weight (V, D) of x's dtype, grad_bias (V) float32 or None) through
+    ot_joiner_weight_grad; workspace_fill: a byte value the workspace is filled with before
+    the call (its contents must not matter)."""
+    rows, V = grad_logits.shape
+    D = x.shape[1]
+    L = lib()
+    L.ot_joiner_weight_grad_workspace_bytes.restype = ctypes.c_size_t
+    nbytes = L.ot_joiner_weight_grad_workspace_bytes(ctypes.c_int64(rows), ctypes.c_int32(V), ctypes.c_int32(D))
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+    if workspace_fill is not None:
+        ws.fill_(workspace_fill)
+    gw = torch.full((V, D), float("nan"), dtype=x.dtype, device=x.device)
+    gb = torch.full((V,), float("nan"), dtype=torch.float32, device=x.device) if want_bias else None
+    check(L.ot_joiner_weight_grad(ptr(grad_logits), ptr(x), ctypes.c_int32(DTYPE[x.dtype]),
+                                  ctypes.c_int64(rows), ctypes.c_int32(V), ctypes.c_int32(D), ptr(ws),
+                                  ctypes.c_size_t(nbytes), ptr(gw), ptr(gb), stream()))
+    return gw, gb
+
+
 def log_probs_given_den(logits, den, targets, U, splits, blank):
     rows, V = logits.shape
     lp = torch.full((rows, 2), float("nan"), dtype=torch.float32, device=logits.device)

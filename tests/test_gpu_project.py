@@ -7,6 +7,8 @@ and gives the scale of a float32 accumulation's rounding error; logits stored in
 2-byte type may in addition be off by one rounding of that type.  The denominators
 are checked against the log-sum-exp of the values the kernel itself stored, which is
 what the loss's own denominator pass would compute from them."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -95,16 +97,17 @@ def test_log_probs_given_denominators(dtype, device):
     assert (got[m] == want[m]).all() and np.isneginf(got[~m]).all()
 
 
+@pytest.mark.parametrize("V", [90, 96])   # 96: this package's weight-gradient kernel; 90: torch's products
 @pytest.mark.parametrize("f32_logits", [True, False])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-def test_python_pipeline_matches_the_unfused_one(dtype, f32_logits, device):
+def test_python_pipeline_matches_the_unfused_one(dtype, f32_logits, V, device):
     """project_joiner + transducer_loss(denominators=...) against torch's linear followed
     by transducer_loss on the same (rounded) logits: same loss, same gradients."""
     import optimized_transducer_amd as ot
     dt = HALF[dtype]
     rng = np.random.default_rng(17)
     T, U, tg, _ = helpers.random_batch(rng, 6, 12, 7, 8)
-    rows, D, V = int((T * (U + 1)).sum()), 64, 90
+    rows, D = int((T * (U + 1)).sum()), 64
     tg = (tg % (V - 1) + 1).astype(np.int32)
     x0, w0, b0 = _inputs(rng, rows, D, V, dt, device)
     dT, dU, dtg = (torch.from_numpy(a).to(device) for a in (T, U, tg))
@@ -224,3 +227,121 @@ def test_denominators_argument_is_checked(device):
     with pytest.raises(RuntimeError, match="multiple of 64"):
         ot.project_joiner(torch.zeros(4, 32, dtype=torch.bfloat16, device=device),
                           torch.zeros(5, 32, dtype=torch.bfloat16, device=device))
+
+
+# ---- backward of the projection in its parameters (ot_joiner_weight_grad)
+def _weight_grad_inputs(rng, rows, V, D, dt, device):
+    # a gradient of logits looks like this: small, mostly one sign per column, a few large entries
+    g = rng.standard_normal((rows, V)) * 0.05 + 0.01
+    g[rng.integers(0, rows, max(rows // 7, 1)), rng.integers(0, V, max(rows // 7, 1))] -= 1.0
+    x = np.tanh(rng.standard_normal((rows, D)))
+    return (torch.from_numpy(g.astype(np.float32)).to(dt).to(device),
+            torch.from_numpy(x.astype(np.float32)).to(dt).to(device))
+
+
+def _check_weight_grad(g, x, gw, gb):
+    want_w, mag_w, want_b, mag_b = oracle.project_joiner_weight_grad(g.float().cpu().numpy(),
+                                                                    x.float().cpu().numpy())
+    got_w = gw.float().cpu().numpy().astype(np.float64)
+    # float32 accumulation in slices (error relative to the sum of the absolute terms) and one
+    # rounding to the 2-byte type
+    tol = 2e-6 * mag_w + ULP[gw.dtype] * np.abs(want_w) * 1.001 + 1e-30
+    assert not np.isnan(got_w).any()
+    assert (np.abs(got_w - want_w) <= tol).all(), (np.abs(got_w - want_w) / tol).max()
+    if gb is not None:
+        got_b = gb.cpu().numpy().astype(np.float64)
+        assert (np.abs(got_b - want_b) <= 2e-6 * mag_b + 1e-30).all(), np.abs(got_b - want_b).max()
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("rows,V,D", [
+    (1, 8, 8), (100, 8, 8), (1000, 24, 64), (31, 504, 512), (5000, 504, 512),
+    # several tiles either way, the last ones partly outside the matrix
+    (3333, 264, 520), (257, 1032, 72), (600, 520, 1032),
+    # fewer rows than slices; one row more than a whole number of stages per slice
+    (40, 128, 64), (64 * 32 + 1, 40, 64),
+    # many rows, narrow matrices
+    (300001, 16, 24)])
+def test_weight_and_bias_gradient_of_the_projection(rows, V, D, dtype, device):
+    rng = np.random.default_rng(rows + 3 * V + D)
+    dt = HALF[dtype]
+    g, x = _weight_grad_inputs(rng, rows, V, D, dt, device)
+    gw, gb = cabi.joiner_weight_grad(g, x, workspace_fill=0xFF)   # workspace full of NaN patterns
+    _check_weight_grad(g, x, gw, gb)
+    # same bits again, whatever the workspace holds; the bias gradient is optional
+    gw2, none = cabi.joiner_weight_grad(g, x, want_bias=False, workspace_fill=0x7F)
+    assert none is None and torch.equal(gw.view(torch.int16), gw2.view(torch.int16))
+    gw3, gb3 = cabi.joiner_weight_grad(g, x)
+    assert torch.equal(gw.view(torch.int16), gw3.view(torch.int16)) and torch.equal(gb, gb3)
+
+
+def test_weight_gradient_is_linear_and_sees_every_row(device):
+    """Properties no tolerance hides: a single nonzero row of g anywhere in the batch gives
+    exactly g[r]^T x[r] rounded once (products of two 2-byte numbers are exact in float32);
+    g of zeros gives zeros; swapping two rows of both operands changes nothing but the
+    order of a float32 sum."""
+    rng = np.random.default_rng(5)
+    rows, V, D = 70000, 72, 136
+    dt = torch.bfloat16
+    g, x = _weight_grad_inputs(rng, rows, V, D, dt, device)
+    zero = torch.zeros_like(g)
+    gw, gb = cabi.joiner_weight_grad(zero, x)
+    assert not gw.float().any() and not gb.any()
+    for r in (0, 31, 32, 1093, 34999, 69999):
+        one = torch.zeros_like(g)
+        one[r] = g[r]
+        gw, gb = cabi.joiner_weight_grad(one, x)
+        want = (g[r].float()[:, None] * x[r].float()[None, :]).to(dt)
+        assert torch.equal(gw.view(torch.int16), want.view(torch.int16)), r
+        assert torch.equal(gb, g[r].float()), r
+
+
+def test_weight_gradient_refuses_what_it_cannot_run(device):
+    L = cabi.lib()
+    L.ot_joiner_weight_grad_workspace_bytes.restype = ctypes.c_size_t
+    g = torch.zeros((64, 16), dtype=torch.bfloat16, device=device)
+    x = torch.zeros((64, 8), dtype=torch.bfloat16, device=device)
+    out = torch.zeros((16, 8), dtype=torch.bfloat16, device=device)
+    n = L.ot_joiner_weight_grad_workspace_bytes(ctypes.c_int64(64), ctypes.c_int32(16), ctypes.c_int32(8))
+    ws = torch.zeros(n, dtype=torch.uint8, device=device)
+
+    def call(g_=g, x_=x, dtype=2, rows=64, V=16, D=8, ws_=ws, n_=n, out_=out):
+        return L.ot_joiner_weight_grad(cabi.ptr(g_), cabi.ptr(x_), ctypes.c_int32(dtype), ctypes.c_int64(rows),
+                                       ctypes.c_int32(V), ctypes.c_int32(D), cabi.ptr(ws_), ctypes.c_size_t(n_),
+                                       cabi.ptr(out_), cabi.ptr(None), cabi.stream())
+    assert call() == 0
+    assert call(dtype=0) == -1 and call(V=12) == -1 and call(D=4) == -1 and call(rows=0) == -1
+    assert call(n_=n - 4) == -1 and call(g_=None) == -1 and call(ws_=None) == -1
+    assert call(g_=g.view(-1)[1:]) == -3 and call(ws_=ws[4:], n_=n) == -3
+    assert L.ot_joiner_weight_grad_workspace_bytes(ctypes.c_int64(0), ctypes.c_int32(16), ctypes.c_int32(8)) == 0
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_backward_of_project_joiner_uses_the_weight_gradient_kernel(dtype, device):
+    """project_joiner's gradients of weight and bias against torch's own backward of the
+    same linear layer on the same incoming gradient, padded vocabulary included."""
+    import optimized_transducer_amd as ot
+    rng = np.random.default_rng(41)
+    dt = HALF[dtype]
+    rows, D, V = 900, 128, 500
+    x0, w0, b0 = _inputs(rng, rows, D, V, dt, device)
+    for vocab_multiple, Vout in ((None, V), (32, 512), (8, 504)):
+        gl = torch.from_numpy((rng.standard_normal((rows, Vout)) * 0.05).astype(np.float32)).to(dt).to(device)
+        gl[:, V:] = 0.0    # what the loss hands back in masked columns
+        x, w, b = (t.clone().requires_grad_(True) for t in (x0, w0, b0))
+        ext = ot._optimized_transducer
+        ext.set_profiling(True)
+        ext.take_profile()
+        logits, _ = ot.project_joiner(x, w, b, float32_logits=False, vocab_multiple=vocab_multiple)
+        logits.backward(gl)
+        names = [n for n, _ in ext.take_profile()]
+        ext.set_profiling(False)
+        # V = 500 itself is not a multiple of 8: torch's products; 504 and 512 are
+        assert ("joiner_weight_grad" in names) == (Vout % 8 == 0 and vocab_multiple is not None), names
+        want_w, mag_w, want_b, mag_b = oracle.project_joiner_weight_grad(
+            gl[:, :V].float().cpu().numpy(), x0.float().cpu().numpy())
+        got_w = w.grad.float().cpu().numpy().astype(np.float64)
+        assert w.grad.shape == (V, D) and b.grad.shape == (V,) and b.grad.dtype == b0.dtype
+        assert (np.abs(got_w - want_w) <= 2e-6 * mag_w + ULP[dt] * np.abs(want_w) * 1.001 + 1e-30).all()
+        assert (np.abs(b.grad.cpu().numpy() - want_b) <= 2e-6 * mag_b + 1e-30).all()
+        assert x.grad.shape == (rows, D)

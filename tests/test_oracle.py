@@ -423,3 +423,32 @@ def test_project_joiner_oracle_is_the_linear_layer_of_the_readme():
     assert np.array_equal(eye, x)
     zero, zmag = oracle.project_joiner(np.zeros((3, 6)), w, b)
     assert np.array_equal(zero, np.tile(b, (3, 1))) and np.array_equal(zmag, np.tile(np.abs(b), (3, 1)))
+
+
+def test_project_joiner_weight_grad_oracle_is_autograds_linear_backward():
+    """Pinned against torch's float64 autograd through nn.functional.linear, against
+    explicit sums on single entries, and by cases that a transposed operand or a sum over
+    the wrong axis would break (one-hot gradient: grad_weight picks a row of x; x of ones:
+    every column of grad_weight is grad_bias)."""
+    rng = np.random.default_rng(29)
+    x = rng.standard_normal((9, 6))
+    w = rng.standard_normal((4, 6))
+    b = rng.standard_normal(4)
+    g = rng.standard_normal((9, 4))
+    gw, gw_mag, gb, gb_mag = oracle.project_joiner_weight_grad(g, x)
+    tw = torch.tensor(w, requires_grad=True)
+    tb = torch.tensor(b, requires_grad=True)
+    torch.nn.functional.linear(torch.tensor(x), tw, tb).backward(torch.tensor(g))
+    assert gw.shape == (4, 6) and np.allclose(gw, tw.grad.numpy(), rtol=1e-14, atol=1e-14)
+    assert gb.shape == (4,) and np.allclose(gb, tb.grad.numpy(), rtol=1e-14, atol=1e-14)
+    for v, k in ((0, 0), (3, 5), (2, 1)):
+        terms = [g[r, v] * x[r, k] for r in range(9)]
+        assert abs(gw[v, k] - sum(terms)) < 1e-13
+        assert abs(gw_mag[v, k] - sum(abs(t) for t in terms)) < 1e-13
+    assert np.allclose(gb_mag, np.abs(g).sum(0))
+    onehot = np.zeros((9, 4))
+    onehot[5, 2] = 1.0
+    ow, _, ob, _ = oracle.project_joiner_weight_grad(onehot, x)
+    assert np.array_equal(ow[2], x[5]) and not ow[[0, 1, 3]].any() and np.array_equal(ob, [0, 0, 1, 0])
+    cw, _, cb, _ = oracle.project_joiner_weight_grad(g, np.ones((9, 6)))
+    assert np.allclose(cw, np.tile(cb[:, None], (1, 6)), rtol=1e-14, atol=1e-14)
