@@ -15,7 +15,7 @@
 // slice of the packed rows; the waves form a 2 x 2 grid, a wave holds 128 x 128 of the tile
 // in 16 accumulator tiles (256 accumulator registers: one workgroup per compute unit).  g
 // and x stream through LDS in stages of 32 rows (two buffers, one barrier per stage); the
-// global loads of a stage are issued three stages ahead into a ring of registers.  The
+// global loads of a stage are issued four stages ahead into a ring of registers.  The
 // workgroup that owns the first 256 columns of D also adds up its g tile by columns for
 // grad_b, in the registers the tile passes through on its way to LDS.  The four tiles of a
 // slice run on the same XCD at the same time, so that its L2 serves the second reader of
@@ -41,7 +41,7 @@ constexpr int kWgPitch = kWgTile + 32;  // LDS row pitch in elements: 144 dwords
                                         // transposing read fall into 4 different quarters of the 64 banks
 constexpr int kWgThreads = 256;
 constexpr int kWgPieces = kWgRows * kWgTile / 8 / kWgThreads;  // 16-byte pieces per thread and operand: 4
-constexpr int kWgAhead = 3;             // stages of global loads in flight
+constexpr int kWgAhead = 4;             // stages of global loads in flight
 
 template <class E>
 __device__ __forceinline__ wg_f32x16 wg_mfma(wg_i16x8 a, wg_i16x8 b, wg_f32x16 c);
@@ -105,34 +105,39 @@ __global__ __launch_bounds__(kWgThreads) void joiner_weight_grad_kernel(
   const unsigned x_stage = x_ok ? (unsigned)(kWgRows * D) * 2u : 0u;
 
   u32x4 gq[kWgAhead][kWgPieces], xq[kWgAhead][kWgPieces];
-  auto issue = [&](u32x4(&gr)[kWgPieces], u32x4(&xr)[kWgPieces]) {
-#pragma unroll
-    for (int i = 0; i < kWgPieces; ++i) {
-      gr[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(g_buf, g_off + i * g_step, 0, 0));
+  // load t of a stage: piece t / 2 of g (t even) or x (t odd)
+  auto issue = [&](u32x4(&gr)[kWgPieces], u32x4(&xr)[kWgPieces], int t) {
+    const int i = t >> 1;
+    if (t & 1)
       xr[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(x_buf, x_off + i * x_step, 0, 0));
+    else
+      gr[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(g_buf, g_off + i * g_step, 0, 0));
+    if (t == 2 * kWgPieces - 1) {
+      g_off += g_stage;
+      x_off += x_stage;
     }
-    g_off += g_stage;
-    x_off += x_stage;
   };
-  // piece t / 2 of g (t even) or x (t odd) into LDS; the g pieces are also added up by
-  // columns for grad_b, rows ascending (only the workgroup of the first tile of D keeps the
-  // sums; adding unconditionally keeps the loop free of branches)
+  // piece t / 2 of g (t even) or x (t odd) into LDS
+  auto deposit = [&](const u32x4(&gr)[kWgPieces], const u32x4(&xr)[kWgPieces], int buf, int t) {
+    const int i = t >> 1;
+    if (t & 1)
+      *reinterpret_cast<u32x4 *>(&s_x[buf][prow + 8 * i][pcol]) = xr[i];
+    else
+      *reinterpret_cast<u32x4 *>(&s_g[buf][prow + 8 * i][pcol]) = gr[i];
+  };
+  // column sums of g for grad_b from the same registers, rows ascending: part t adds the
+  // two columns of dword t % 4 of piece t / 4.  Only the workgroup of the first tile of D
+  // keeps the sums; all of them add, which keeps the loop free of branches (sharing the
+  // pieces among the workgroups that load the same tile of g, with a branch around each
+  // part, was measured and is slower).
   float bsum[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) bsum[e] = 0.f;
-  auto deposit = [&](const u32x4(&gr)[kWgPieces], const u32x4(&xr)[kWgPieces], int buf, int t) {
-    const int i = t >> 1;
-    if (t & 1) {
-      *reinterpret_cast<u32x4 *>(&s_x[buf][prow + 8 * i][pcol]) = xr[i];
-    } else {
-      *reinterpret_cast<u32x4 *>(&s_g[buf][prow + 8 * i][pcol]) = gr[i];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const unsigned w = gr[i][e];
-        bsum[2 * e] += to_float<E>((unsigned short)(w & 0xFFFFu));
-        bsum[2 * e + 1] += to_float<E>((unsigned short)(w >> 16));
-      }
-    }
+  auto add_up = [&](const u32x4(&gr)[kWgPieces], int t) {
+    const int e = t & 3;
+    const unsigned w = gr[t >> 2][e];
+    bsum[2 * e] += to_float<E>((unsigned short)(w & 0xFFFFu));
+    bsum[2 * e + 1] += to_float<E>((unsigned short)(w >> 16));
   };
 
   // operands of a k-step (16 rows): a[i] for the 4 tiles of g, b[j] for the 4 tiles of x,
@@ -161,9 +166,13 @@ __global__ __launch_bounds__(kWgThreads) void joiner_weight_grad_kernel(
   // stages 0 .. kWgAhead-1 on their way, stage 0 in LDS, its first k-step in registers
   wg_i16x4 fa[4][2], fb[4][2], na[4][2], nb[4][2];
 #pragma unroll
-  for (int a = 0; a < kWgAhead; ++a) issue(gq[a], xq[a]);
+  for (int a = 0; a < kWgAhead; ++a)
+#pragma unroll
+    for (int t = 0; t < 2 * kWgPieces; ++t) issue(gq[a], xq[a], t);
 #pragma unroll
   for (int t = 0; t < 2 * kWgPieces; ++t) deposit(gq[0], xq[0], 0, t);
+#pragma unroll
+  for (int t = 0; t < 4 * kWgPieces; ++t) add_up(gq[0], t);
   lds_barrier();
 #pragma unroll
   for (int r = 0; r < 16; ++r) fetch(fa, fb, 0, 0, r);
@@ -171,11 +180,11 @@ __global__ __launch_bounds__(kWgThreads) void joiner_weight_grad_kernel(
   // One wave per SIMD: whatever the wave waits for, the matrix core waits for too.  So
   // everything else is dealt out over the 32 products of a stage by hand, and the fences
   // keep the compiler from gathering it again:
-  //   products of k-step 0 | the global loads of stage s + kWgAhead (three stages to arrive),
+  //   products of k-step 0 | the global loads of stage s + kWgAhead (over three stages to arrive),
   //                        | the 16 operand reads of k-step 1
   //   products of k-step 1 | stage s + 1 into the other LDS buffer (its readers passed the
-  //                        | previous barrier), the barrier, the operand reads of stage
-  //                        | s + 1's k-step 0
+  //                        | previous barrier) and into the column sums, the barrier, the
+  //                        | operand reads of stage s + 1's k-step 0
   // The stages are rounded up to a multiple of kWgAhead: a stage behind the slice's end
   // loads zeros and adds zeros.
   for (int s = 0; s < nstages; s += kWgAhead) {
@@ -185,7 +194,7 @@ __global__ __launch_bounds__(kWgThreads) void joiner_weight_grad_kernel(
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
         acc[t >> 2][t & 3] = wg_mfma<E>(wg_join(fa[t >> 2]), wg_join(fb[t & 3]), acc[t >> 2][t & 3]);
-        if (t == 0) issue(gq[a], xq[a]);
+        if (t < 2 * kWgPieces) issue(gq[a], xq[a], t);
         fetch(na, nb, cur, 1, t);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -193,6 +202,7 @@ __global__ __launch_bounds__(kWgThreads) void joiner_weight_grad_kernel(
       for (int t = 0; t < 16; ++t) {
         acc[t >> 2][t & 3] = wg_mfma<E>(wg_join(na[t >> 2]), wg_join(nb[t & 3]), acc[t >> 2][t & 3]);
         if (t < 8) deposit(gq[(a + 1) % kWgAhead], xq[(a + 1) % kWgAhead], nxt, t);
+        add_up(gq[(a + 1) % kWgAhead], t);
         if (t == 7) lds_barrier();
         if (t >= 8) {
           fetch(fa, fb, nxt, 0, 2 * (t - 8));

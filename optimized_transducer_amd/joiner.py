@@ -123,9 +123,12 @@ class ProjectJoinerFunction(torch.autograd.Function):
         x, weight = ctx.saved_tensors
         V = ctx.V
         g = grad_logits if grad_logits.dtype == x.dtype else grad_logits.to(x.dtype)
-        # grad_x: a product with the contraction index running fastest in memory on one
-        # side, the kind the library's kernels are good at
-        grad_x = g @ weight if ctx.needs_input_grad[0] else None
+        # grad_x = g W by the library, handed W^T (a copy of the small weight) so that the
+        # contraction index runs fastest in both operands: its kernel for that layout is
+        # the faster one here (0.53 against 0.64 ms at 752 k rows, V = D = 512)
+        grad_x = None
+        if ctx.needs_input_grad[0]:
+            grad_x = torch.nn.functional.linear(g, weight.t().contiguous())
         want_w = ctx.needs_input_grad[1]
         want_b = ctx.has_bias and ctx.needs_input_grad[2]
         grad_w = grad_b = None
