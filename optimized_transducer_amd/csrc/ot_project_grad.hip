@@ -79,7 +79,8 @@ __global__ __launch_bounds__(kWgThreads) void joiner_weight_grad_kernel(
   __shared__ __attribute__((aligned(16))) unsigned short s_g[2][kWgRows][kWgPitch];
   __shared__ __attribute__((aligned(16))) unsigned short s_x[2][kWgRows][kWgPitch];
   __shared__ float s_b[kWgThreads / 32][kWgTile];
-  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles = m_tiles * n_tiles;
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
@@ -179,34 +180,42 @@ __global__ __launch_bounds__(kWgThreads) void joiner_weight_grad_kernel(
 
   // One wave per SIMD: whatever the wave waits for, the matrix core waits for too.  So
   // everything else is dealt out over the 32 products of a stage by hand, and the fences
-  // keep the compiler from gathering it again:
-  //   products of k-step 0 | the global loads of stage s + kWgAhead (over three stages to arrive),
-  //                        | the 16 operand reads of k-step 1
-  //   products of k-step 1 | stage s + 1 into the other LDS buffer (its readers passed the
-  //                        | previous barrier) and into the column sums, the barrier, the
-  //                        | operand reads of stage s + 1's k-step 0
-  // The stages are rounded up to a multiple of kWgAhead: a stage behind the slice's end
-  // loads zeros and adds zeros.
+  // keep the compiler from gathering it again.  The four waves run in step (one barrier per
+  // stage) and share the compute unit's address path (a global load: 16 clocks) and LDS
+  // write port (16 bytes per lane: 13 clocks), so loads and LDS writes are spread over the
+  // whole stage rather than bunched behind consecutive products:
+  //   global load t of stage s + kWgAhead     after product 4 t             (t = 0 .. 7)
+  //   piece t of stage s + 1 into LDS         after product 3 t             (t = 0 .. 7)
+  //   operand reads of k-step 1               after products 0 .. 15, one each
+  //   column sums of stage s + 1              after products 16 .. 31
+  //   the barrier                             after product 23
+  //   operand reads of stage s + 1, k-step 0  after products 24 .. 31, two each
+  // The copies go to the other LDS buffer, whose readers passed the previous barrier.  The
+  // stages are rounded up to a multiple of kWgAhead: a stage behind the slice's end loads
+  // zeros and adds zeros.
   for (int s = 0; s < nstages; s += kWgAhead) {
 #pragma unroll
     for (int a = 0; a < kWgAhead; ++a) {
       const int cur = (s + a) & 1, nxt = cur ^ 1;
 #pragma unroll
-      for (int t = 0; t < 16; ++t) {
-        acc[t >> 2][t & 3] = wg_mfma<E>(wg_join(fa[t >> 2]), wg_join(fb[t & 3]), acc[t >> 2][t & 3]);
-        if (t < 2 * kWgPieces) issue(gq[a], xq[a], t);
-        fetch(na, nb, cur, 1, t);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-#pragma unroll
-      for (int t = 0; t < 16; ++t) {
-        acc[t >> 2][t & 3] = wg_mfma<E>(wg_join(na[t >> 2]), wg_join(nb[t & 3]), acc[t >> 2][t & 3]);
-        if (t < 8) deposit(gq[(a + 1) % kWgAhead], xq[(a + 1) % kWgAhead], nxt, t);
-        add_up(gq[(a + 1) % kWgAhead], t);
-        if (t == 7) lds_barrier();
-        if (t >= 8) {
-          fetch(fa, fb, nxt, 0, 2 * (t - 8));
-          fetch(fa, fb, nxt, 0, 2 * (t - 8) + 1);
+      for (int slot = 0; slot < 32; ++slot) {
+        const int t = slot & 15;
+        if (slot < 16)
+          acc[t >> 2][t & 3] = wg_mfma<E>(wg_join(fa[t >> 2]), wg_join(fb[t & 3]), acc[t >> 2][t & 3]);
+        else
+          acc[t >> 2][t & 3] = wg_mfma<E>(wg_join(na[t >> 2]), wg_join(nb[t & 3]), acc[t >> 2][t & 3]);
+        if (slot % 4 == 0) issue(gq[a], xq[a], slot / 4);
+        if (slot % 3 == 0 && slot / 3 < 2 * kWgPieces)
+          deposit(gq[(a + 1) % kWgAhead], xq[(a + 1) % kWgAhead], nxt, slot / 3);
+        if (slot < 16) {
+          fetch(na, nb, cur, 1, t);
+        } else {
+          add_up(gq[(a + 1) % kWgAhead], t);
+          if (slot == 23) lds_barrier();
+          if (slot >= 24) {
+            fetch(fa, fb, nxt, 0, 2 * (slot - 24));
+            fetch(fa, fb, nxt, 0, 2 * (slot - 24) + 1);
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
