@@ -182,6 +182,8 @@ def project_joiner(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
       ``bias`` come from this package's own kernel when V is a multiple of 8 (one pass over
       the gradient of the logits and ``x``, float32 accumulation, the same bits on every
       run), the gradient of ``x`` from torch's product; ``denominators`` carries no gradient.
+      With float32 logits their gradient is rounded to the dtype of ``x`` first, for all
+      three products (as autograd does for a Linear layer under autocast).
     """
     if vocab_multiple is not None and (not isinstance(vocab_multiple, int) or vocab_multiple < 1):
         raise ValueError("project_joiner: vocab_multiple must be a positive integer or None, "
