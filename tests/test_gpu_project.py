@@ -275,6 +275,22 @@ def test_weight_and_bias_gradient_of_the_projection(rows, V, D, dtype, device):
     assert torch.equal(gw.view(torch.int16), gw3.view(torch.int16)) and torch.equal(gb, gb3)
 
 
+def test_weight_gradient_on_random_shapes(device):
+    """Shapes nobody picked: rows around the slice and stage boundaries, V and D any multiples of 8."""
+    rng = np.random.default_rng(2024)
+    for trial in range(24):
+        V = 8 * int(rng.integers(1, 140))
+        D = 8 * int(rng.integers(1, 140))
+        rows = int(rng.choice([rng.integers(1, 70), rng.integers(70, 3000), 64 * 32 * int(rng.integers(1, 4)) + int(rng.integers(-2, 3))]))
+        dt = (torch.float16, torch.bfloat16)[trial % 2]
+        g, x = _weight_grad_inputs(rng, rows, V, D, dt, device)
+        gw, gb = cabi.joiner_weight_grad(g, x, workspace_fill=0xFF)
+        try:
+            _check_weight_grad(g, x, gw, gb)
+        except AssertionError as e:
+            raise AssertionError("rows = %d, V = %d, D = %d, %s: %s" % (rows, V, D, dt, e))
+
+
 def test_weight_gradient_is_linear_and_sees_every_row(device):
     """Properties no tolerance hides: a single nonzero row of g anywhere in the batch gives
     exactly g[r]^T x[r] rounded once (products of two 2-byte numbers are exact in float32);
