@@ -413,6 +413,22 @@ int ot_joiner_project(const void *x, const void *weight, const float *bias,
                       void *logits, int32_t logits_dtype, float *den,
                       void *stream);
 
+/* ot_joiner_project for a caller that lends a workspace of
+ * ot_joiner_project_workspace_bytes(rows, V) bytes (4-byte aligned; contents
+ * irrelevant before and after; 0 bytes for V <= 256).  With it, the 256-column
+ * passes over the vocabulary of one block of rows run side by side on
+ * workgroups of one XCD instead of one after the other on one workgroup, so
+ * that x leaves HBM once whatever V is; every pass leaves a partial
+ * log-sum-exp per row in the workspace and a second kernel merges them in pass
+ * order.  Same logits, bit for bit; den from the same stored values with its
+ * terms grouped by pass.  A NULL or short workspace falls back to
+ * ot_joiner_project. */
+size_t ot_joiner_project_workspace_bytes(int64_t rows, int32_t V);
+int ot_joiner_project_ws(const void *x, const void *weight, const float *bias,
+                         int32_t dtype, int64_t rows, int32_t D, int32_t V,
+                         void *logits, int32_t logits_dtype, float *den,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
 /* Backward of that projection with respect to its parameters (no counterpart
  * in the reference either: there autograd's Linear does it, README.md:176-177
  * with the loss's gradient of cuda.cu:471-489 as input):

@@ -791,12 +791,18 @@ std::pair<torch::Tensor, torch::Tensor> joiner_project(const torch::Tensor &x,
   torch::Tensor logits =
       torch::empty({rows, V}, x.options().dtype(float32_logits ? torch::kFloat : x.scalar_type()));
   torch::Tensor den = torch::empty({rows}, x.options().dtype(torch::kFloat));
+  // room for one partial log-sum-exp per row and 256-column pass: with it the passes of a
+  // block of rows run side by side on one XCD and x is read from HBM once
+  const size_t ws_bytes = ot_joiner_project_workspace_bytes(rows, (int32_t)V);
+  torch::Tensor workspace;
+  if (ws_bytes > 0) workspace = torch::empty({(int64_t)ws_bytes}, x.options().dtype(torch::kUInt8));
   {
     ScopedTimer timer("joiner_project", stream);
-    OT_CHECK(ot_joiner_project(x.data_ptr(), weight.data_ptr(),
-                               b.defined() ? b.data_ptr<float>() : nullptr, dtype, rows, (int32_t)D,
-                               (int32_t)V, logits.data_ptr(), float32_logits ? OT_DTYPE_F32 : dtype,
-                               den.data_ptr<float>(), stream));
+    OT_CHECK(ot_joiner_project_ws(x.data_ptr(), weight.data_ptr(),
+                                  b.defined() ? b.data_ptr<float>() : nullptr, dtype, rows, (int32_t)D,
+                                  (int32_t)V, logits.data_ptr(), float32_logits ? OT_DTYPE_F32 : dtype,
+                                  den.data_ptr<float>(), ws_bytes > 0 ? workspace.data_ptr() : nullptr,
+                                  ws_bytes, stream));
   }
   return {logits, den};
 }

@@ -84,7 +84,7 @@ template <class E, bool OUT_F32, int SV>
 __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
     const unsigned short *__restrict__ x, const unsigned short *__restrict__ w,
     const float *__restrict__ bias, int64_t rows, int D, int V, void *__restrict__ logits,
-    float *__restrict__ den) {
+    float *__restrict__ den, int paired) {
   __shared__ __attribute__((aligned(16))) unsigned char s_stage[2 * kProjStageBytes];
   __shared__ float2 s_part[2][kProjRows];
   __shared__ __attribute__((aligned(16))) float s_bias[kProjCols];  // the pass's starting values
@@ -93,10 +93,26 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int c = lane & 31, h = lane >> 5;
-  // Persistent workgroups: workgroup g takes the 128-row tiles g, g + gridDim.x, ...;
-  // the loads of the next tile's first stages are already in flight while the current
-  // tile's last pass is stored.
+  // Persistent workgroups: workgroup g takes the 128-row tiles g, g + gridDim.x, ... and
+  // all passes of each; the loads of the next tile's first stages are already in flight
+  // while the current tile's last pass is stored.
+  // Paired (the caller lends room for one partial log-sum-exp per row and pass): a workgroup
+  // takes ONE pass of its tiles, and the workgroups that take the other passes of the same
+  // tiles run beside it on the same XCD (ids 8 apart), so that x leaves HBM once and the
+  // other readers are served by that XCD's L2; `den` then holds the parts, pass-major.
   const int64_t ntiles = (rows + kProjRows - 1) / kProjRows;
+  const int npasses_all = (V + kProjCols - 1) / kProjCols;
+  int64_t tile_first = blockIdx.x, tile_stride = gridDim.x;
+  int pass_first = 0, pass_count = npasses_all;
+  if (paired) {
+    const int k = (int)blockIdx.x >> 3;
+    pass_first = k % npasses_all;
+    pass_count = 1;
+    tile_first = (int64_t)(k / npasses_all) * 8 + (blockIdx.x & 7);
+    tile_stride = (int64_t)(gridDim.x / 8 / npasses_all) * 8;
+    den += (int64_t)pass_first * rows;
+  }
+  const int pass_end = pass_first + pass_count;
   // the weight and the bias as raw buffers: vocabulary entries past V read as zeros
   const __amdgpu_buffer_rsrc_t wbuf = make_buffer(w, (unsigned)V * (unsigned)D * 2u);
   const __amdgpu_buffer_rsrc_t bbuf = make_buffer(bias ? bias : den, bias ? (unsigned)V * 4u : 0u);
@@ -127,14 +143,13 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
   }
 
   const int ksteps = D / kProjK;
-  const int npasses = (V + kProjCols - 1) / kProjCols;
 
   // global loads run two stages ahead of the matrix work
   // Loads past the last stage are issued all the same (W reads as zeros there, x is
   // re-read): with a branch around them the number of loads in flight would not be
   // known at compile time and every wait would have to drain them all.
-  int64_t load_tile = blockIdx.x;
-  int load_pass = 0, load_kk = 0;
+  int64_t load_tile = tile_first;
+  int load_pass = pass_first, load_kk = 0;
   __amdgpu_buffer_rsrc_t xbuf = x_tile(load_tile);
   auto load_stage = [&](ProjStage &st) {
     const unsigned wbase =
@@ -148,9 +163,9 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
           xbuf, piece_src, (unsigned)(load_kk * kProjK) * 2u + q * piece_src_step, 0);
     if (++load_kk == ksteps) {
       load_kk = 0;
-      if (++load_pass == npasses) {
-        load_pass = 0;
-        load_tile += gridDim.x;
+      if (++load_pass == pass_end) {
+        load_pass = pass_first;
+        load_tile += tile_stride;
         xbuf = x_tile(load_tile);
       }
     }
@@ -191,19 +206,19 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
     const float b = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, (unsigned)v * 4u, 0, 0));
     return v < V ? b : OT_NEG_INF;
   };
-  s_bias[tid] = starting_value(tid);
+  s_bias[tid] = starting_value(pass_first * kProjCols + tid);
   load_stage(set_a);
   load_stage(set_b);
   store_stage(set_a, 0);
   load_stage(set_a);
-  for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+  for (int64_t tile = tile_first; tile < ntiles; tile += tile_stride) {
   const int64_t row0 = tile * kProjRows;
   const unsigned nrows = (unsigned)min((int64_t)kProjRows, rows - row0);
   // stores to rows past the array vanish
   const __amdgpu_buffer_rsrc_t obuf =
       make_buffer(static_cast<char *>(logits) + row0 * V * kOutBytes, nrows * (unsigned)V * kOutBytes);
   float m_run[2] = {OT_NEG_INF, OT_NEG_INF}, s_run[2] = {0.f, 0.f};
-  for (int pass = 0; pass < npasses; ++pass) {
+  for (int pass = pass_first; pass < pass_end; ++pass) {
     const int n0 = pass * kProjCols + 128 * wn;  // first column of this wave in the pass
     // accumulators start from the bias: tile (rs, vt), register 4 j + i holds vocabulary
     // entry n0 + 32 vt + 8 j + 4 h + i of packed row 64 wm + 32 rs + c.  The pass's
@@ -241,7 +256,7 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
     unsigned char *tile = s_tile + wave * kProjTileBytes;
     // starting values of the next pass (of the next tile after the last one), fetched
     // before this pass's stores are issued
-    if (npasses > 1) s_bias[tid] = starting_value((pass + 1 < npasses ? pass + 1 : 0) * kProjCols + tid);
+    if (pass_count > 1) s_bias[tid] = starting_value((pass + 1 < pass_end ? pass + 1 : pass_first) * kProjCols + tid);
     constexpr int kTilePitch = OUT_F32 ? kProjTilePitch : kProjTilePitch / 2 + 8;  // 144 / 80 bytes
     constexpr int kLanesPerRow = OUT_F32 ? 8 : 4;        // 16 bytes per lane
     constexpr int kRowsPerStore = kWave / kLanesPerRow;  // 8 or 16
@@ -348,9 +363,25 @@ __global__ __launch_bounds__(kProjThreads, 2) void joiner_project_kernel(
 
 static inline int launch_status() { return (int)hipGetLastError(); }
 
+// den[r] = log-sum-exp of a row's parts (one per pass over the vocabulary), parts in order
+__global__ __launch_bounds__(kBlock) void project_den_merge_kernel(const float *__restrict__ parts,
+                                                                  int nparts, int64_t rows,
+                                                                  float *__restrict__ den) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r >= rows) return;
+  float m = OT_NEG_INF;
+  for (int k = 0; k < nparts; ++k) m = fmaxf(m, parts[(int64_t)k * rows + r]);
+  const float ref = __builtin_isinf(m) ? 0.f : m;
+  float sum = 0.f;
+  for (int k = 0; k < nparts; ++k) sum += expf(parts[(int64_t)k * rows + r] - ref);
+  den[r] = logf(sum) + ref;
+}
+
+// Workgroups of a launch, and whether the passes of a tile can be dealt out to workgroups of
+// one XCD (`parts`: room for rows * passes floats, or NULL).
 template <class E, bool OUT_F32>
 static int launch_project(const unsigned short *x, const unsigned short *w, const float *bias,
-                          int64_t rows, int32_t D, int32_t V, void *logits, float *den,
+                          int64_t rows, int32_t D, int32_t V, void *logits, float *den, float *parts,
                           hipStream_t s) {
   // two resident workgroups per compute unit walk over the 128-row tiles
   int device = 0, cus = 0;
@@ -358,14 +389,22 @@ static int launch_project(const unsigned short *x, const unsigned short *w, cons
       hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
     return OT_E_BAD_ARG;
   const int64_t tiles = (rows + kProjRows - 1) / kProjRows;
-  const int64_t blocks = tiles < 2 * (int64_t)cus ? tiles : 2 * (int64_t)cus;
+  const int npasses = (V + kProjCols - 1) / kProjCols;
+  int64_t blocks = tiles < 2 * (int64_t)cus ? tiles : 2 * (int64_t)cus;
+  // paired walk: every XCD's share of the resident workgroups splits evenly over the passes
+  // and there is at least one tile for every group of them
+  const int64_t resident = 2 * (int64_t)cus / 8 * 8;
+  const bool paired = parts && npasses > 1 && resident > 0 && (resident / 8) % npasses == 0 &&
+                      tiles * npasses >= resident;
+  if (paired) blocks = resident;
+  float *const den_out = paired ? parts : den;
   const unsigned esize = OUT_F32 ? 4u : 2u;
   int sv = (int)(16u / esize);  // elements per store
   while (sv > 1 && (V % sv != 0 || (reinterpret_cast<uintptr_t>(logits) & (uintptr_t)(sv * esize - 1))))
     sv >>= 1;
 #define OT_LAUNCH_PROJ(SV_)                                                                       \
   hipLaunchKernelGGL((joiner_project_kernel<E, OUT_F32, SV_>), dim3((unsigned)blocks), dim3(kProjThreads), \
-                     0, s, x, w, bias, rows, D, V, logits, den)
+                     0, s, x, w, bias, rows, D, V, logits, den_out, paired ? 1 : 0)
   switch (sv) {
     case 8: if constexpr (!OUT_F32) { OT_LAUNCH_PROJ(8); } break;
     case 4: OT_LAUNCH_PROJ(4); break;
@@ -373,6 +412,9 @@ static int launch_project(const unsigned short *x, const unsigned short *w, cons
     default: OT_LAUNCH_PROJ(1); break;
   }
 #undef OT_LAUNCH_PROJ
+  if (paired)
+    hipLaunchKernelGGL(project_den_merge_kernel, dim3((unsigned)((rows + kBlock - 1) / kBlock)), dim3(kBlock),
+                       0, s, parts, npasses, rows, den);
   return launch_status();
 }
 
@@ -382,9 +424,9 @@ using namespace ot;
 
 extern "C" {
 
-int ot_joiner_project(const void *x, const void *weight, const float *bias, int32_t dtype,
-                      int64_t rows, int32_t D, int32_t V, void *logits, int32_t logits_dtype,
-                      float *den, void *stream) {
+static int joiner_project_checked(const void *x, const void *weight, const float *bias, int32_t dtype,
+                                  int64_t rows, int32_t D, int32_t V, void *logits, int32_t logits_dtype,
+                                  float *den, float *parts, void *stream) {
   if (!x || !weight || !logits || !den || rows <= 0 || rows > INT32_MAX || D <= 0 || V <= 0 ||
       (dtype != OT_DTYPE_F16 && dtype != OT_DTYPE_BF16) ||
       (logits_dtype != OT_DTYPE_F32 && logits_dtype != dtype))
@@ -396,6 +438,7 @@ int ot_joiner_project(const void *x, const void *weight, const float *bias, int3
     return OT_E_BAD_ARG;
   if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(weight) & 15) ||
       (reinterpret_cast<uintptr_t>(bias) & 15) || (reinterpret_cast<uintptr_t>(den) & 3) ||
+      (reinterpret_cast<uintptr_t>(parts) & 3) ||
       (reinterpret_cast<uintptr_t>(logits) & (logits_dtype == OT_DTYPE_F32 ? 3 : 1)))
     return OT_E_MISALIGNED;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -403,11 +446,32 @@ int ot_joiner_project(const void *x, const void *weight, const float *bias, int3
   const unsigned short *wp = static_cast<const unsigned short *>(weight);
   if (dtype == OT_DTYPE_BF16)
     return logits_dtype == OT_DTYPE_F32
-               ? launch_project<BF16, true>(xp, wp, bias, rows, D, V, logits, den, s)
-               : launch_project<BF16, false>(xp, wp, bias, rows, D, V, logits, den, s);
+               ? launch_project<BF16, true>(xp, wp, bias, rows, D, V, logits, den, parts, s)
+               : launch_project<BF16, false>(xp, wp, bias, rows, D, V, logits, den, parts, s);
   return logits_dtype == OT_DTYPE_F32
-             ? launch_project<F16, true>(xp, wp, bias, rows, D, V, logits, den, s)
-             : launch_project<F16, false>(xp, wp, bias, rows, D, V, logits, den, s);
+             ? launch_project<F16, true>(xp, wp, bias, rows, D, V, logits, den, parts, s)
+             : launch_project<F16, false>(xp, wp, bias, rows, D, V, logits, den, parts, s);
+}
+
+int ot_joiner_project(const void *x, const void *weight, const float *bias, int32_t dtype,
+                      int64_t rows, int32_t D, int32_t V, void *logits, int32_t logits_dtype,
+                      float *den, void *stream) {
+  return joiner_project_checked(x, weight, bias, dtype, rows, D, V, logits, logits_dtype, den, nullptr, stream);
+}
+
+size_t ot_joiner_project_workspace_bytes(int64_t rows, int32_t V) {
+  if (rows <= 0 || V <= kProjCols) return 0;
+  return (size_t)((V + kProjCols - 1) / kProjCols) * (size_t)rows * sizeof(float);
+}
+
+int ot_joiner_project_ws(const void *x, const void *weight, const float *bias, int32_t dtype,
+                         int64_t rows, int32_t D, int32_t V, void *logits, int32_t logits_dtype,
+                         float *den, void *workspace, size_t workspace_bytes, void *stream) {
+  float *parts = static_cast<float *>(workspace);
+  if (!parts || workspace_bytes < ot_joiner_project_workspace_bytes(rows, V) ||
+      ot_joiner_project_workspace_bytes(rows, V) == 0)
+    parts = nullptr;
+  return joiner_project_checked(x, weight, bias, dtype, rows, D, V, logits, logits_dtype, den, parts, stream);
 }
 
 int ot_log_probs_given_den(const void *logits, int32_t dtype, const float *den,

@@ -272,12 +272,24 @@ def gradient_half(logits, lp, den, alpha, beta, targets, T, U, splits, blank, fr
 ANY_DTYPE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 
-def joiner_project(x, weight, bias, out_dtype, logits=None):
+def joiner_project(x, weight, bias, out_dtype, logits=None, workspace=False):
+    """ot_joiner_project, or with workspace=True ot_joiner_project_ws on a workspace full of
+    NaN patterns."""
     rows, D = x.shape
     V = weight.shape[0]
     if logits is None:
         logits = torch.full((rows, V), float("nan"), dtype=out_dtype, device=x.device)
     den = torch.full((rows,), float("nan"), dtype=torch.float32, device=x.device)
+    if workspace:
+        L = lib()
+        L.ot_joiner_project_workspace_bytes.restype = ctypes.c_size_t
+        nbytes = L.ot_joiner_project_workspace_bytes(ctypes.c_int64(rows), ctypes.c_int32(V))
+        ws = torch.full((max(nbytes, 4),), 0xFF, dtype=torch.uint8, device=x.device)
+        check(L.ot_joiner_project_ws(ptr(x), ptr(weight), ptr(bias), ctypes.c_int32(DTYPE[x.dtype]),
+                                     ctypes.c_int64(rows), ctypes.c_int32(D), ctypes.c_int32(V),
+                                     ptr(logits), ctypes.c_int32(ANY_DTYPE[out_dtype]), ptr(den),
+                                     ptr(ws if nbytes else None), ctypes.c_size_t(nbytes), stream()))
+        return logits, den
     check(lib().ot_joiner_project(ptr(x), ptr(weight), ptr(bias), ctypes.c_int32(DTYPE[x.dtype]),
                                   ctypes.c_int64(rows), ctypes.c_int32(D), ctypes.c_int32(V),
                                   ptr(logits), ctypes.c_int32(ANY_DTYPE[out_dtype]), ptr(den),

@@ -43,6 +43,12 @@ def _check(x, w, b, out_dtype):
     ref = m + np.log(np.exp(got - m[:, None]).sum(1))
     d = den.cpu().numpy().astype(np.float64)
     assert (np.abs(d - ref) <= 4e-7 * np.maximum(np.abs(ref), np.abs(m)) + 1e-6).all(), np.abs(d - ref).max()
+    # with a workspace (passes side by side, partial log-sum-exps merged): the same logits bit
+    # for bit, denominators of the same stored values
+    logits_ws, den_ws = cabi.joiner_project(x, w, b, out_dtype, workspace=True)
+    assert torch.equal(logits_ws.view(torch.uint8), logits.view(torch.uint8))
+    d = den_ws.cpu().numpy().astype(np.float64)
+    assert (np.abs(d - ref) <= 4e-7 * np.maximum(np.abs(ref), np.abs(m)) + 1e-6).all(), np.abs(d - ref).max()
     return logits, den
 
 
@@ -51,7 +57,8 @@ def _check(x, w, b, out_dtype):
 @pytest.mark.parametrize("rows,D,V", [(700, 64, 500), (256, 64, 128), (1, 512, 37), (513, 192, 1030),
                                       (300, 128, 6), (64, 256, 130),
                                       # more 128-row tiles than resident workgroups: some take two
-                                      (70001, 64, 40), (66000, 64, 300),
+                                      # (and, with a workspace, the passes run side by side)
+                                      (70001, 64, 40), (66000, 64, 300), (40000, 64, 1030), (33000, 128, 520),
                                       # many passes over the vocabulary, long rows of x
                                       (300, 128, 5000), (200, 1024, 777)])
 def test_projection_and_denominators(rows, D, V, dtype, out, device):
