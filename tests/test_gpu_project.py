@@ -236,6 +236,35 @@ def test_denominators_argument_is_checked(device):
                           torch.zeros(5, 32, dtype=torch.bfloat16, device=device))
 
 
+def test_projection_workspace_is_optional(device):
+    """ot_joiner_project_ws without a workspace, or with one that is too short, is
+    ot_joiner_project; a vocabulary of one pass needs none."""
+    L = cabi.lib()
+    L.ot_joiner_project_workspace_bytes.restype = ctypes.c_size_t
+    rng = np.random.default_rng(3)
+    rows, D, V = 70000, 64, 600
+    assert L.ot_joiner_project_workspace_bytes(ctypes.c_int64(rows), ctypes.c_int32(256)) == 0
+    assert L.ot_joiner_project_workspace_bytes(ctypes.c_int64(rows), ctypes.c_int32(257)) == 2 * rows * 4
+    n = L.ot_joiner_project_workspace_bytes(ctypes.c_int64(rows), ctypes.c_int32(V))
+    assert n == 3 * rows * 4
+    x, w, b = _inputs(rng, rows, D, V, torch.bfloat16, device)
+    want, want_den = cabi.joiner_project(x, w, b, torch.bfloat16)
+    ws = torch.zeros(n, dtype=torch.uint8, device=device)
+    for ws_ptr, ws_bytes in ((None, 0), (ws, n - 4), (None, n)):
+        logits = torch.full((rows, V), float("nan"), dtype=torch.bfloat16, device=device)
+        den = torch.full((rows,), float("nan"), dtype=torch.float32, device=device)
+        cabi.check(L.ot_joiner_project_ws(cabi.ptr(x), cabi.ptr(w), cabi.ptr(b), ctypes.c_int32(2),
+                                          ctypes.c_int64(rows), ctypes.c_int32(D), ctypes.c_int32(V),
+                                          cabi.ptr(logits), ctypes.c_int32(2), cabi.ptr(den), cabi.ptr(ws_ptr),
+                                          ctypes.c_size_t(ws_bytes), cabi.stream()))
+        assert torch.equal(logits.view(torch.int16), want.view(torch.int16)) and torch.equal(den, want_den)
+    # same argument checks as ot_joiner_project
+    rc = L.ot_joiner_project_ws(cabi.ptr(x), cabi.ptr(w), cabi.ptr(b), ctypes.c_int32(0), ctypes.c_int64(rows),
+                                ctypes.c_int32(D), ctypes.c_int32(V), cabi.ptr(want), ctypes.c_int32(2),
+                                cabi.ptr(want_den), cabi.ptr(ws), ctypes.c_size_t(n), cabi.stream())
+    assert rc == -1
+
+
 # ---- backward of the projection in its parameters (ot_joiner_weight_grad)
 def _weight_grad_inputs(rng, rows, V, D, dt, device):
     # a gradient of logits looks like this: small, mostly one sign per column, a few large entries
