@@ -59,6 +59,8 @@ def _check(x, w, b, out_dtype):
                                       # more 128-row tiles than resident workgroups: some take two
                                       # (and, with a workspace, the passes run side by side)
                                       (70001, 64, 40), (66000, 64, 300), (40000, 64, 1030), (33000, 128, 520),
+                                      # four and eight passes side by side
+                                      (40000, 64, 1000), (50000, 64, 2048),
                                       # many passes over the vocabulary, long rows of x
                                       (300, 128, 5000), (200, 1024, 777)])
 def test_projection_and_denominators(rows, D, V, dtype, out, device):
